@@ -1,0 +1,161 @@
+// Host API: argument checks, Split_K policy and the two launches behind
+// SpMM_SplitK_API (reference csrc/SpMM_API.cu:55-130), plus the C++ wrappers
+// that keep the reference's compressor signatures (build/SpMM_API.cuh:51-58).
+#include "SpMM_API.h"
+#include "flashllm_spmm.h"
+#include "spmm_launch.h"
+
+#include <cstdio>
+#include <cstdlib>
+
+namespace {
+
+// The N values the reference dispatches on (csrc/SpMM_API.cu:79-118).
+bool supported_n(int n)
+{
+    return n == 8 || n == 16 || n == 32 || n == 64 || (n > 0 && n % 128 == 0);
+}
+
+int check_shape(const void* comp, const int* offs, const void* b, const void* c, int m, int n, int k, const void* ws, int split_k)
+{
+    if (!comp || !offs || !b || !c)
+        return hipErrorInvalidValue;
+    if (m <= 0 || k <= 0 || m % 128 || k % 64 || split_k < 1)
+        return hipErrorInvalidValue;
+    if (!supported_n(n)) {
+        std::printf("MM_Sparse_API Error: Unsupported N dimension %d!\n", n);
+        return hipErrorUnknown;
+    }
+    if (split_k > 1 && !ws)
+        return hipErrorInvalidValue;
+    if (reinterpret_cast<uintptr_t>(comp) % 16 || reinterpret_cast<uintptr_t>(b) % 16 || reinterpret_cast<uintptr_t>(c) % 8
+        || reinterpret_cast<uintptr_t>(ws) % 16)
+        return hipErrorInvalidValue;
+    return hipSuccess;
+}
+
+}  // namespace
+
+extern "C" {
+
+int flashllm_spmm_partials(void*       stream,
+                           const void* comp,
+                           const int*  offs,
+                           const void* b,
+                           void*       c,
+                           int         m,
+                           int         n,
+                           int         k,
+                           void*       ws,
+                           int         split_k)
+{
+    const int bad = check_shape(comp, offs, b, c, m, n, k, ws, split_k);
+    if (bad)
+        return bad;
+    return flashllm_hip_launch_spmm(stream, comp, offs, b, split_k == 1 ? c : ws, m, n, k, split_k);
+}
+
+int flashllm_splitk_reduce(void* stream, void* c, const void* ws, int m, int n, int split_k)
+{
+    if (!c || !ws || m <= 0 || n <= 0 || split_k < 1 || (static_cast<long>(m) * n) % 8)
+        return hipErrorInvalidValue;
+    return flashllm_hip_launch_reduce(stream, c, ws, static_cast<long>(m) * n, split_k);
+}
+
+int flashllm_spmm_splitk(void*       stream,
+                         const void* /*A: unused, as in the reference*/,
+                         const void* comp,
+                         const int*  offs,
+                         const void* b,
+                         void*       c,
+                         int         m,
+                         int         n,
+                         int         k,
+                         void*       ws,
+                         int         split_k)
+{
+    int rc = flashllm_spmm_partials(stream, comp, offs, b, c, m, n, k, ws, split_k);
+    if (rc || split_k == 1)
+        return rc;
+    return flashllm_hip_launch_reduce(stream, c, ws, static_cast<long>(m) * n, split_k);
+}
+
+size_t flashllm_workspace_bytes(int m, int n, int split_k)
+{
+    if (split_k <= 1 || m <= 0 || n <= 0)
+        return 0;
+    return static_cast<size_t>(split_k) * m * n * sizeof(uint16_t);
+}
+
+// One wave streams one (row tile, K slice, column group) and owns 16 KB of
+// LDS, so a CU holds about eight of them; the grid should put roughly that
+// many on each of the 256 CUs, in slices of equal length.
+int flashllm_splitk_heuristic(int m, int n, int k)
+{
+    if (m <= 0 || k <= 0 || n <= 0 || m % 128 || k % 64)
+        return 1;
+    const int  kt         = k / 64;
+    const int  col_groups = n <= 64 ? 1 : n / 64;
+    const long units      = static_cast<long>(m / 128) * col_groups;
+    const long target     = 256L * 8;
+    int        best       = 1;
+    double     best_cost  = 1e30;
+    for (int s = 1; s <= kt && s <= 32; s++) {
+        const int  avg   = (kt - 1) / s + 1;  // longest slice, in k tiles
+        const long waves = units * s;
+        // time ~ rounds of resident waves x longest slice, plus slab traffic
+        const long   rounds = (waves + target - 1) / target;
+        const double stream = static_cast<double>(rounds) * avg;
+        const double slabs  = s > 1 ? 0.04 * s * kt / 8.0 : 0.0;
+        const double idle   = waves < target ? static_cast<double>(target - waves) / target * avg * 0.5 : 0.0;
+        const double cost   = stream + slabs + idle;
+        if (cost < best_cost) {
+            best_cost = cost;
+            best      = s;
+        }
+    }
+    return best;
+}
+
+}  // extern "C"
+
+hipError_t SpMM_SplitK_API(hipStream_t  stream,
+                           const half*  A,
+                           const uint4* Compressed_A,
+                           const int*   TileOffsets,
+                           const half*  B,
+                           half*        C,
+                           const int    M_Global,
+                           const int    N_Global,
+                           const int    K_Global,
+                           half*        Reduction_Workspace,
+                           int          Split_K)
+{
+    return static_cast<hipError_t>(flashllm_spmm_splitk(
+        stream, A, Compressed_A, TileOffsets, B, C, M_Global, N_Global, K_Global, Reduction_Workspace, Split_K));
+}
+
+namespace {
+int init_or_exit(int rc)
+{
+    if (rc == FLASHLLM_E_NOMEM) {
+        std::printf("InitSparseMatrixA: Error in malloc memory from host memory!\n");
+        std::exit(-1);
+    }
+    if (rc < 0)
+        std::fprintf(stderr, "InitSparseMatrixA: rejected (code %d): M must be a multiple of 128 and K of 64\n", rc);
+    return rc;
+}
+}  // namespace
+
+int InitSparseMatrixA_API(half* A_h, int M, int /*N*/, int K, uint32_t** Compressed_A, int** TileOffsets)
+{
+    return init_or_exit(
+        flashllm_init_sparse_matrix_a(reinterpret_cast<const uint16_t*>(A_h), M, K, Compressed_A, TileOffsets));
+}
+
+int InitSparseMatrixA_API_NoReorder(half* A_h, int M, int /*N*/, int K, uint32_t** Compressed_A, int** TileOffsets)
+{
+    return init_or_exit(flashllm_init_sparse_matrix_a_noreorder(
+        reinterpret_cast<const uint16_t*>(A_h), M, K, Compressed_A, TileOffsets));
+}

@@ -1,0 +1,29 @@
+// The thin extern "C" HIP layer underneath the host API: one function per
+// kernel launch, nothing but pointers and ints, no validation (the host API
+// has checked the shapes these grids assume).
+#ifndef FLASHLLM_AMD_SPMM_LAUNCH_H
+#define FLASHLLM_AMD_SPMM_LAUNCH_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+// out: C when split_k == 1, else the slab workspace (split_k * M * N halfs).
+// Requires M % 128 == 0, K % 64 == 0, N in {8,16,32,64} or N % 64 == 0.
+int flashllm_hip_launch_spmm(void*       stream,
+                             const void* compressed_a,
+                             const int*  tile_offsets,
+                             const void* b,
+                             void*       out,
+                             int         m,
+                             int         n,
+                             int         k,
+                             int         split_k);
+
+// c[e] = rn16(sum_s float(ws[s*mn + e])); requires mn % 8 == 0.
+int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws, long mn, int split_k);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

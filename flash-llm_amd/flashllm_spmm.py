@@ -1,0 +1,180 @@
+"""ctypes binding of libSpMM_API.so's plain-C entry points (include/flashllm_spmm.h).
+
+Thin by design: every call goes straight into the shared library.  There is
+no CPU fallback; if the library is missing, loading raises.  Device buffers
+are torch tensors (torch is only the allocator and the stream provider).
+
+The functions mirror the reference's API (build/SpMM_API.cuh:38-67):
+init_sparse_matrix_a <-> InitSparseMatrixA_API, spmm_splitk <-> SpMM_SplitK_API,
+gen_sparse_matrix_bin_file <-> GenSparseMatrixBinFile.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libSpMM_API.so")
+
+_lib = None
+
+_u16p = ctypes.POINTER(ctypes.c_uint16)
+_u32p = ctypes.POINTER(ctypes.c_uint32)
+_i32p = ctypes.POINTER(ctypes.c_int)
+_vp = ctypes.c_void_p
+
+# name -> (restype, argtypes); every symbol include/flashllm_spmm.h declares
+SIGNATURES = {
+    "flashllm_init_sparse_matrix_a": (ctypes.c_int, [_u16p, ctypes.c_int, ctypes.c_int, ctypes.POINTER(_u32p), ctypes.POINTER(_i32p)]),
+    "flashllm_init_sparse_matrix_a_noreorder": (ctypes.c_int, [_u16p, ctypes.c_int, ctypes.c_int, ctypes.POINTER(_u32p), ctypes.POINTER(_i32p)]),
+    "flashllm_free": (None, [_vp]),
+    "flashllm_set_compress_threads": (None, [ctypes.c_int]),
+    "flashllm_spmm_splitk": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int]),
+    "flashllm_spmm_partials": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int]),
+    "flashllm_splitk_reduce": (ctypes.c_int, [_vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "flashllm_splitk_heuristic": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "flashllm_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "flashllm_gen_sparse_matrix_bin_file": (ctypes.c_int, [ctypes.c_char_p, ctypes.c_int, ctypes.c_int, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_char_p]),
+    "GenSparseMatrixBinFile": (None, [ctypes.c_char_p, ctypes.c_int, ctypes.c_int, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_char_p]),
+}
+
+
+def lib():
+    """Loads libSpMM_API.so once.  Raises OSError when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise OSError(f"{LIB_PATH} is not built: run `make -C {_HERE}` (or __graft_entry__.build())")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+class CompressError(ValueError):
+    def __init__(self, code):
+        super().__init__(f"Tiled-CSL compression failed with code {code}")
+        self.code = code
+
+
+def _compress(fn_name, a, threads):
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.float16:
+        a = a.view(np.uint16)
+    if a.dtype != np.uint16 or a.ndim != 2:
+        raise TypeError("A must be a 2-D float16 (or uint16 bit pattern) array")
+    m, k = a.shape
+    L = lib()
+    if threads is not None:
+        L.flashllm_set_compress_threads(int(threads))
+    comp = _u32p()
+    offs = _i32p()
+    n = getattr(L, fn_name)(a.ctypes.data_as(_u16p), m, k, ctypes.byref(comp), ctypes.byref(offs))
+    if n < 0:
+        raise CompressError(n)
+    try:
+        offsets = np.ctypeslib.as_array(offs, shape=(n,)).copy()
+        nnz = int(offsets[n - 1]) * 4
+        items = np.ctypeslib.as_array(comp, shape=(max(nnz, 1),))[:nnz].copy()
+    finally:
+        L.flashllm_free(comp)
+        L.flashllm_free(offs)
+    return items, offsets
+
+
+def init_sparse_matrix_a(a, threads=None):
+    """InitSparseMatrixA_API: (Compressed_A uint32[NNZ_padded], TileOffsets int32[tiles+2])."""
+    return _compress("flashllm_init_sparse_matrix_a", a, threads)
+
+
+def init_sparse_matrix_a_noreorder(a, threads=None):
+    """InitSparseMatrixA_API_NoReorder."""
+    return _compress("flashllm_init_sparse_matrix_a_noreorder", a, threads)
+
+
+def splitk_heuristic(m, n, k):
+    return lib().flashllm_splitk_heuristic(m, n, k)
+
+
+def workspace_bytes(m, n, split_k):
+    return lib().flashllm_workspace_bytes(m, n, split_k)
+
+
+def gen_sparse_matrix_bin_file(dense, m, k, nz, offsets, sizes):
+    rc = lib().flashllm_gen_sparse_matrix_bin_file(dense.encode(), m, k, nz.encode(), offsets.encode(), sizes.encode())
+    if rc:
+        raise CompressError(rc)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _stream(stream):
+    import torch
+
+    s = stream if stream is not None else torch.cuda.current_stream()
+    return ctypes.c_void_p(s.cuda_stream)
+
+
+class HipError(RuntimeError):
+    def __init__(self, code):
+        super().__init__(f"libSpMM_API returned hipError_t {code}")
+        self.code = code
+
+
+def spmm_splitk(comp, offs, b, c, m, n, k, workspace, split_k, stream=None, a=None):
+    """SpMM_SplitK_API on torch device tensors; asynchronous on `stream`
+    (default: torch's current stream).  Raises HipError on a non-zero code."""
+    rc = lib().flashllm_spmm_splitk(_stream(stream), _ptr(a), _ptr(comp), _ptr(offs), _ptr(b), _ptr(c), m, n, k, _ptr(workspace), split_k)
+    if rc:
+        raise HipError(rc)
+
+
+def spmm_partials(comp, offs, b, c, m, n, k, workspace, split_k, stream=None):
+    rc = lib().flashllm_spmm_partials(_stream(stream), _ptr(comp), _ptr(offs), _ptr(b), _ptr(c), m, n, k, _ptr(workspace), split_k)
+    if rc:
+        raise HipError(rc)
+
+
+def splitk_reduce(c, workspace, m, n, split_k, stream=None):
+    rc = lib().flashllm_splitk_reduce(_stream(stream), _ptr(c), _ptr(workspace), m, n, split_k)
+    if rc:
+        raise HipError(rc)
+
+
+class SparseWeight:
+    """A compressed weight resident on the GPU: what a caller keeps per linear
+    layer (the reference's DenseWeight::NZWeights/TileOffsets/SplitK fields,
+    third_party/ft.patch:456-462)."""
+
+    def __init__(self, a_host, split_k=None, reorder=True, device="cuda"):
+        import torch
+
+        a_host = np.ascontiguousarray(a_host)
+        self.m, self.k = a_host.shape
+        fn = init_sparse_matrix_a if reorder else init_sparse_matrix_a_noreorder
+        items, offsets = fn(a_host)
+        self.nnz = items.size
+        self.num_offsets = offsets.size
+        if items.size == 0:  # fully sparse: keep one addressable element, as the reference's callers do
+            items = np.zeros(4, dtype=np.uint32)
+        self.comp = torch.from_numpy(items.view(np.int32)).to(device)
+        self.offs = torch.from_numpy(offsets).to(device)
+        self.split_k = split_k
+        self.device = device
+
+    def matmul(self, b, n, c=None, workspace=None, split_k=None, stream=None):
+        """b: fp16 device tensor holding column-major K x N; returns column-major M x N."""
+        import torch
+
+        s = split_k or self.split_k or splitk_heuristic(self.m, n, self.k)
+        if c is None:
+            c = torch.empty(n * self.m, dtype=torch.float16, device=self.device)
+        if s > 1 and workspace is None:
+            workspace = torch.empty(s * n * self.m, dtype=torch.float16, device=self.device)
+        spmm_splitk(self.comp, self.offs, b, c, self.m, n, self.k, workspace, s, stream=stream)
+        return c

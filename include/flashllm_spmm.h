@@ -1,0 +1,115 @@
+/*
+ * Plain-C ABI of libSpMM_API.so: the same hot path as SpMM_API.h with
+ * nothing but pointers and ints in the signatures, for callers that bind
+ * over an FFI.  Every function returns instead of exiting.
+ */
+#ifndef FLASHLLM_AMD_SPMM_C_H
+#define FLASHLLM_AMD_SPMM_C_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Error codes of the host-side functions (negative return values). */
+#define FLASHLLM_E_SHAPE (-1)   /* M % 128 != 0, K % 64 != 0 or not positive */
+#define FLASHLLM_E_NOMEM (-2)   /* host allocation failed */
+#define FLASHLLM_E_NOZERO (-3)  /* padding needed in a bank with no zero position */
+#define FLASHLLM_E_ARG (-5)     /* null pointer */
+#define FLASHLLM_E_IO (-6)      /* file could not be opened / short read */
+
+/*
+ * C twin of InitSparseMatrixA_API (reference csrc/SpMM_API.cu:163-360).
+ * A_h: row-major M x K fp16 bit patterns on the host.  On success returns
+ * (M/128)*(K/64)+2 and sets *Compressed_A / *TileOffsets to buffers that
+ * must be released with flashllm_free.
+ */
+int flashllm_init_sparse_matrix_a(const uint16_t* A_h, int M, int K, uint32_t** Compressed_A, int** TileOffsets);
+
+/* C twin of InitSparseMatrixA_API_NoReorder (reference csrc/SpMM_API.cu:363-489). */
+int flashllm_init_sparse_matrix_a_noreorder(
+    const uint16_t* A_h, int M, int K, uint32_t** Compressed_A, int** TileOffsets);
+
+/* Releases a buffer returned by the two functions above (the reference's
+ * callers use free(), kernel_benchmark/spmm_test.cu:268-269). */
+void flashllm_free(void* p);
+
+/* Worker threads the compressors use (tiles are independent); 0 = one per
+ * host core, capped at 16.  The reference is single-threaded
+ * (csrc/SpMM_API.cu:235-351); the bytes do not depend on this setting. */
+void flashllm_set_compress_threads(int n);
+
+/*
+ * C twin of SpMM_SplitK_API (reference csrc/SpMM_API.cu:55-130).  stream is
+ * a hipStream_t (NULL = the default stream); all other pointers are device
+ * pointers.  Returns the hipError_t as an int (0 = success).
+ */
+int flashllm_spmm_splitk(void*       stream,
+                         const void* A,
+                         const void* Compressed_A,
+                         const int*  TileOffsets,
+                         const void* B,
+                         void*       C,
+                         int         M,
+                         int         N,
+                         int         K,
+                         void*       Reduction_Workspace,
+                         int         Split_K);
+
+/*
+ * The first half of flashllm_spmm_splitk alone (reference
+ * csrc/SpMM_API.cu:73-118): launches only the SpMM kernel and leaves the
+ * Split_K fp16 slabs in Reduction_Workspace (or writes C when Split_K == 1).
+ * For callers that time the kernels separately or fuse the reduction.
+ */
+int flashllm_spmm_partials(void*       stream,
+                           const void* Compressed_A,
+                           const int*  TileOffsets,
+                           const void* B,
+                           void*       C,
+                           int         M,
+                           int         N,
+                           int         K,
+                           void*       Reduction_Workspace,
+                           int         Split_K);
+
+/* The second half alone (reference csrc/Reduction_Kernel.cuh:24-45, launch
+ * csrc/SpMM_API.cu:126-128): C[e] = rn16(sum_s float(ws[s*M*N + e])). */
+int flashllm_splitk_reduce(void* stream, void* C, const void* Reduction_Workspace, int M, int N, int Split_K);
+
+/*
+ * Split_K recommended for one MI355X (256 CUs, wave64).  Takes the place of
+ * the per-shape tables hand-tuned for A100 in the reference
+ * (kernel_benchmark/benchmark.sh:13-15,
+ * end2end_inference/ft_tools/huggingface_opt_convert_Phase2.py:20).
+ */
+int flashllm_splitk_heuristic(int M, int N, int K);
+
+/* Bytes the caller must provide as Reduction_Workspace (0 when Split_K == 1);
+ * the contract of reference build/SpMM_API.cuh:33-36. */
+size_t flashllm_workspace_bytes(int M, int N, int Split_K);
+
+/* Six-argument file exporter (reference csrc/SpMM_API.cu:500-555) that
+ * returns 0 or a FLASHLLM_E_* code instead of exiting. */
+int flashllm_gen_sparse_matrix_bin_file(const char* DenseMatrixFileName,
+                                        int         M,
+                                        int         K,
+                                        const char* NZWeightsFileName,
+                                        const char* TileOffsetsFileName,
+                                        const char* OutputSizesFileName);
+
+/* Same symbol and signature as the reference's only extern "C" export
+ * (csrc/SpMM_API.cu:500-505); exits on error like the reference. */
+void GenSparseMatrixBinFile(char* DenseMatrixFileName,
+                            int   M,
+                            int   K,
+                            char* NZWeightsFileName,
+                            char* TileOffsetsFileName,
+                            char* OutputSizesFileName);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,93 @@
+"""The C-ABI library loads, exports what the headers declare, and its host-side entry points
+behave like the reference's (no GPU compute here)."""
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+import synth
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_c_symbols():
+    text = open(os.path.join(ROOT, "include", "flashllm_spmm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(flashllm_\w+|GenSparseMatrixBinFile)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported(product):
+    names = declared_c_symbols()
+    assert "flashllm_spmm_splitk" in names and "GenSparseMatrixBinFile" in names and len(names) >= 11
+    assert sorted(product.SIGNATURES) == names
+    L = product.lib()
+    for name in names:
+        assert getattr(L, name) is not None
+
+
+def test_cxx_drop_in_symbols_are_exported(product):
+    out = subprocess.run(["nm", "-D", "--demangle", product.LIB_PATH], check=True, capture_output=True, text=True).stdout
+    for sig in ("SpMM_SplitK_API(ihipStream_t*, __half const*, HIP_vector_type<unsigned int, 4u> const*, int const*, __half const*, __half*, int, int, int, __half*, int)",
+                "InitSparseMatrixA_API(__half*, int, int, int, unsigned int**, int**)",
+                "InitSparseMatrixA_API_NoReorder(__half*, int, int, int, unsigned int**, int**)"):
+        assert re.search(r" T " + re.escape(sig), out), sig
+    assert re.search(r" T GenSparseMatrixBinFile$", out, flags=re.M)
+
+
+def test_spmm_rejects_bad_arguments_before_any_launch(product):
+    L = product.lib()
+    ok = 0x1000  # fake, suitably aligned device addresses: validation must fail before they are used
+    INVALID, UNKNOWN = 1, 999  # hipErrorInvalidValue, hipErrorUnknown
+    call = lambda **kw: L.flashllm_spmm_splitk(None, None, kw.get("comp", ok), kw.get("offs", ok), kw.get("b", ok), kw.get("c", ok),
+                                               kw.get("m", 256), kw.get("n", 16), kw.get("k", 128), kw.get("ws", ok), kw.get("s", 2))
+    assert call(m=100) == INVALID
+    assert call(k=100) == INVALID
+    assert call(s=0) == INVALID
+    assert call(comp=None) == INVALID
+    assert call(b=None) == INVALID
+    assert call(ws=None, s=2) == INVALID
+    assert call(comp=ok + 4) == INVALID
+    assert call(n=24) == UNKNOWN       # the reference prints and returns cudaErrorUnknown for such N
+    assert call(n=192) == UNKNOWN
+    assert L.flashllm_splitk_reduce(None, None, ok, 128, 8, 2) == INVALID
+
+
+def test_workspace_and_heuristic(product):
+    assert product.workspace_bytes(1024, 8, 1) == 0
+    assert product.workspace_bytes(36864, 16, 3) == 3 * 36864 * 16 * 2
+    for m, n, k in [(36864, 16, 9216), (9216, 16, 9216), (9216, 16, 36864), (1024, 8, 1024), (49152, 32, 12288), (128, 64, 64)]:
+        s = product.splitk_heuristic(m, n, k)
+        assert 1 <= s <= min(32, k // 64)
+    assert product.splitk_heuristic(100, 16, 64) == 1
+
+
+def test_bin_file_export(product, oracle, tmp_path):
+    m, k = 256, 192
+    a = synth.sparse_matrix(m, k, 0.8, 21)
+    dense = tmp_path / "w.bin"
+    a.tofile(dense)
+    names = [str(tmp_path / f"w.{x}.bin") for x in ("NZWeights", "TileOffsets", "OutputSizes")]
+    product.gen_sparse_matrix_bin_file(str(dense), m, k, *names)
+    _, items, offsets = oracle.compress_reorder(a)
+    assert np.array_equal(np.fromfile(names[0], dtype=np.uint32), items)
+    assert np.array_equal(np.fromfile(names[1], dtype=np.int32), offsets)
+    assert np.fromfile(names[2], dtype=np.int32).tolist() == [items.size, offsets.size]
+    # the reference's own symbol, as its ctypes caller binds it
+    product.lib().GenSparseMatrixBinFile(str(dense).encode(), m, k, *[n.encode() for n in names])
+    assert np.array_equal(np.fromfile(names[0], dtype=np.uint32), items)
+    with pytest.raises(product.CompressError) as e:
+        product.gen_sparse_matrix_bin_file(str(tmp_path / "missing.bin"), m, k, *names)
+    assert e.value.code == -6
+    with pytest.raises(product.CompressError) as e:  # short file
+        product.gen_sparse_matrix_bin_file(str(dense), m * 2, k, *names)
+    assert e.value.code == -6
+
+
+def test_product_sources_never_touch_the_oracle():
+    pkg = os.path.join(ROOT, "flash-llm_amd")
+    for base, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".cpp", ".hip", ".h", ".py")) or f == "Makefile":
+                assert "oracle" not in open(os.path.join(base, f)).read().lower(), f

@@ -1,0 +1,249 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle.
+
+Tolerance on C (floating point): max|C - ref| / max|ref| <= 1e-2 and element-wise
+|C - ref| <= 1e-2*|ref| + 1e-2*rms(ref), ref = fp32-accumulated product on the decompressed
+weights.  Everything integer (the compressed stream the kernel consumes, the reduction of given
+slabs, exact special cases) is compared bit for bit.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import synth
+from gpu_util import assert_close, errors, run_spmm
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def torch_gpu():
+    import torch
+
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    return torch
+
+
+# --- BASELINE config 1: 1024 x 1024, 80 %, U[-1,1], N = 8, Split_K = 1, seed 0 -----------------
+def test_config1_plumbing(product, oracle, torch_gpu):
+    say("config1 1024x1024 N=8 split_k=1")
+    a = synth.sparse_matrix(1024, 1024, 0.8, 0)
+    b = synth.dense_b(1024, 8, 0)
+    c, w, _ = run_spmm(product, a, b, 8, 1)
+    _, items, offsets = oracle.compress_reorder(a)
+    assert np.array_equal(w.comp.cpu().numpy().view(np.uint32), items)
+    assert np.array_equal(w.offs.cpu().numpy(), offsets)
+    model, ref = oracle.spmm_model(a, b, 8, 1)
+    assert_close(c, ref, "config1")
+    # against the oracle's own fp16 result the difference is summation order only
+    assert np.max(np.abs(c.astype(np.float32) - model.astype(np.float32))) <= 2.0 ** -8 * np.max(np.abs(ref))
+
+
+@pytest.mark.parametrize("n", [8, 16, 32, 64, 128, 256])
+@pytest.mark.parametrize("split_k", [1, 3])
+def test_every_supported_n(product, oracle, torch_gpu, n, split_k):
+    say(f"N sweep n={n} split_k={split_k}")
+    a = synth.sparse_matrix(512, 1024, 0.8, 3)
+    b = synth.dense_b(1024, n, 4)
+    c, _, _ = run_spmm(product, a, b, n, split_k)
+    _, ref = oracle.spmm_model(a, b, n, split_k)
+    assert_close(c, ref, f"n={n} split_k={split_k}")
+
+
+@pytest.mark.parametrize("reorder", [True, False])
+@pytest.mark.parametrize("sparsity", [0.0, 0.3, 0.5, 0.7, 0.9, 0.99, 1.0])
+def test_any_density(product, oracle, torch_gpu, sparsity, reorder):
+    """Tiles denser than 50 % overflow the reference kernel's register budget; here any density works."""
+    say(f"density sparsity={sparsity} reorder={reorder}")
+    a = synth.sparse_matrix(256, 512, sparsity, 5)
+    b = synth.dense_b(512, 16, 6)
+    for split_k in (1, 2):
+        c, _, _ = run_spmm(product, a, b, 16, split_k, reorder=reorder)
+        _, ref = oracle.spmm_model(a, b, 16, split_k)
+        if sparsity == 1.0:
+            assert not c.any()
+        else:
+            assert_close(c, ref, f"sparsity={sparsity} split_k={split_k}")
+
+
+def test_ragged_tiles_and_empty_slices(product, oracle, torch_gpu):
+    """Empty tiles at the start, middle and end of a slice, one-vector tiles, a full tile, and more
+    slices than k tiles."""
+    say("ragged tiles")
+    m, k = 256, 640
+    a = synth.sparse_matrix(m, k, 0.8, 8)
+    a[:128, 0:64] = 0          # first tile of tile row 0 empty
+    a[:128, 256:384] = 0       # two empty tiles in the middle
+    a[128:, 576:640] = 0       # last tile of tile row 1 empty
+    a[128:, 64:128] = 0
+    a[130, 70] = 1.5           # a single nonzero: one vector with three paddings
+    a[:128, 448:512] = synth.sparse_matrix(128, 64, 0.0, 9)  # a full tile
+    b = synth.dense_b(k, 16, 10)
+    for split_k in (1, 2, 5, 10, 16):
+        c, _, _ = run_spmm(product, a, b, 16, split_k)
+        _, ref = oracle.spmm_model(a, b, 16, split_k)
+        assert_close(c, ref, f"ragged split_k={split_k}")
+
+
+def test_ones_matrix_subset_sums(product, oracle, torch_gpu):
+    """The reference benchmark's data (A in {0,1}, B in fifths): small exact sums."""
+    say("ones matrix")
+    m, n, k = 256, 8, 256
+    a = synth.sparse_matrix(m, k, 0.8, 3, dist="ones")
+    b = (np.random.default_rng(0).integers(0, 5, size=(n, k)) / 4 - 0.5).astype(np.float16)  # quarters: exact in fp16/fp32
+    c, _, _ = run_spmm(product, a, b, n, 1)
+    want = (b.astype(np.float32) @ a.astype(np.float32).T).astype(np.float16)
+    assert np.array_equal(c, want)
+
+
+def test_scaled_permutation_exact(product, torch_gpu):
+    say("permutation")
+    k = m = 512
+    perm = np.random.default_rng(1).permutation(k)
+    a = np.zeros((m, k), dtype=np.float16)
+    a[np.arange(m), perm] = 2.0
+    b = synth.dense_b(k, 32, 5)
+    for split_k in (1, 4):
+        c, _, _ = run_spmm(product, a, b, 32, split_k)
+        assert np.array_equal(c, b[:, perm] * np.float16(2.0))
+
+
+def test_special_values_flow_through(product, oracle, torch_gpu):
+    """-0 and NaN in A are dropped by the compressor, so C stays finite; Inf propagates."""
+    say("special values")
+    a = synth.sparse_matrix(128, 128, 0.8, 11)
+    bits = a.view(np.uint16)
+    bits[3, 5] = 0x7E00   # NaN: dropped
+    bits[4, 6] = 0x8000   # -0: dropped
+    b = np.abs(synth.dense_b(128, 8, 12)) + np.float16(0.5)
+    c, _, _ = run_spmm(product, a, b, 8, 1)
+    assert np.all(np.isfinite(c))
+    dec = oracle.scatter(*oracle.compress_reorder(a)[1:], 128, 128).view(np.float16)
+    _, ref = oracle.spmm_model(dec, b, 8, 1)
+    assert_close(c, ref, "specials")
+    bits[7, 9] = 0x7C00   # +Inf: kept
+    c, _, _ = run_spmm(product, a, b, 8, 1)
+    assert np.all(np.isinf(c[:, 7])) and np.all(np.isfinite(np.delete(c, 7, axis=1)))
+
+
+def test_split_k_reduction_bit_exact(product, oracle, torch_gpu):
+    torch = torch_gpu
+    say("reduction kernel")
+    rng = np.random.default_rng(2)
+    for m, n, s in [(128, 8, 2), (1024, 16, 7), (256, 64, 32), (384, 8, 5)]:
+        ws_h = (rng.standard_normal((s, n * m)) * 3).astype(np.float16)
+        ws = torch.from_numpy(ws_h).cuda()
+        c = torch.zeros(n * m, dtype=torch.float16, device="cuda")
+        product.splitk_reduce(c, ws, m, n, s)
+        torch.cuda.synchronize()
+        want = oracle.splitk_reduce(ws_h, n * m, s)
+        assert np.array_equal(c.cpu().numpy().view(np.uint16), want.view(np.uint16))
+
+
+def test_partials_then_reduce_equals_api(product, oracle, torch_gpu):
+    torch = torch_gpu
+    say("partials + reduce")
+    m, n, k, s = 512, 16, 1024, 4
+    a = synth.sparse_matrix(m, k, 0.8, 13)
+    b_h = synth.dense_b(k, n, 14)
+    c_api, w, ws_api = run_spmm(product, a, b_h, n, s)
+    b = torch.from_numpy(b_h).cuda()
+    ws = torch.zeros(s * n * m, dtype=torch.float16, device="cuda")
+    c = torch.zeros(n * m, dtype=torch.float16, device="cuda")
+    product.spmm_partials(w.comp, w.offs, b, c, m, n, k, ws, s)
+    torch.cuda.synchronize()
+    slabs = ws.cpu().numpy().reshape(s, n, m)
+    assert np.array_equal(slabs.view(np.uint16), ws_api.cpu().numpy().reshape(s, n, m).view(np.uint16))
+    for i, (kb, ke) in enumerate(oracle.splitk_ranges(k, s)):
+        _, ref = oracle.spmm_model(np.ascontiguousarray(a[:, kb * 64:ke * 64]), np.ascontiguousarray(b_h[:, kb * 64:ke * 64]), n, 1)
+        assert_close(slabs[i], ref, f"slab {i}")
+    product.splitk_reduce(c, ws, m, n, s)
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy().view(np.uint16), c_api.reshape(-1).view(np.uint16))
+    assert np.array_equal(c_api.reshape(-1).view(np.uint16), oracle.splitk_reduce(slabs.reshape(s, -1), n * m, s).view(np.uint16))
+
+
+def test_runs_on_a_side_stream_and_is_repeatable(product, oracle, torch_gpu):
+    torch = torch_gpu
+    say("side stream")
+    m, n, k, s = 512, 16, 512, 2
+    a = synth.sparse_matrix(m, k, 0.8, 15)
+    b_h = synth.dense_b(k, n, 16)
+    w = product.SparseWeight(a)
+    b = torch.from_numpy(b_h).cuda()
+    ws = torch.empty(s * n * m, dtype=torch.float16, device="cuda")
+    outs = []
+    stream = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    for _ in range(3):
+        c = torch.empty(n * m, dtype=torch.float16, device="cuda")
+        with torch.cuda.stream(stream):
+            w.matmul(b, n, c=c, workspace=ws, split_k=s, stream=stream)
+        stream.synchronize()
+        outs.append(c.cpu().numpy())
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[1], outs[2])
+    _, ref = oracle.spmm_model(a, b_h, n, s)
+    assert_close(outs[0].reshape(n, m), ref, "side stream")
+
+
+# --- BASELINE config 2: 9216 x 9216, 80 %, N = 16, Split_K in {1,2,4,8} -------------------------
+def test_config2_skinny(product, oracle, torch_gpu):
+    say("config2 generate")
+    m = k = 9216
+    a = synth.sparse_matrix(m, k, 0.8, 0)
+    b = synth.dense_b(k, 16, 0)
+    say("config2 oracle compress")
+    _, items, offsets = oracle.compress_reorder(a)
+    ref, _ = oracle.gemm_f32(a, b, 16)
+    for split_k in (1, 2, 4, 8):
+        say(f"config2 split_k={split_k}")
+        c, w, _ = run_spmm(product, a, b, 16, split_k)
+        if split_k == 1:
+            assert np.array_equal(w.comp.cpu().numpy().view(np.uint32), items)
+            assert np.array_equal(w.offs.cpu().numpy(), offsets)
+        assert_close(c, ref, f"config2 split_k={split_k}")
+
+
+# --- the headline shape: 36864 x 9216, 80 %, N(0, 0.02) weights, N(0,1) activations, N = 16 -----
+def test_headline_shape(product, oracle, torch_gpu):
+    m, k, n = 36864, 9216, 16
+    say("headline generate")
+    a = synth.sparse_matrix(m, k, 0.8, 0, dist="normal", sigma=0.02, threads=16)
+    b = synth.dense_b(k, n, 0, dist="normal")
+    say("headline reference gemm")
+    ref, _ = oracle.gemm_f32(a, b, n)
+    s = product.splitk_heuristic(m, n, k)
+    for split_k in sorted({1, 3, s}):
+        say(f"headline split_k={split_k}")
+        c, w, _ = run_spmm(product, a, b, n, split_k)
+        assert_close(c, ref, f"headline split_k={split_k}")
+    say("headline round trip of the compressed stream")
+    back = oracle.scatter(w.comp.cpu().numpy().view(np.uint32)[:w.nnz], w.offs.cpu().numpy(), m, k)
+    bits = a.view(np.uint16)
+    mag = bits & 0x7FFF
+    assert np.array_equal(back, np.where((mag != 0) & (mag <= 0x7C00), bits, 0))
+    # linearity in B (a size-independent property): A(b1 + b2) vs A b1 + A b2
+    b2 = synth.dense_b(k, n, 1, dist="normal")
+    bsum = (b.astype(np.float32) + b2.astype(np.float32)).astype(np.float16)
+    c1, _, _ = run_spmm(product, a, b, n, s)
+    c2, _, _ = run_spmm(product, a, b2, n, s)
+    c12, _, _ = run_spmm(product, a, bsum, n, s)
+    rel, _ = errors(c12, c1.astype(np.float32) + c2.astype(np.float32))
+    assert rel <= 2e-2
+
+
+# --- config 4 flavour: non-uniform rows, N = 32 --------------------------------------------------
+def test_nonuniform_rows(product, oracle, torch_gpu):
+    say("non-uniform rows")
+    m, k, n = 3072, 3072, 32
+    a = synth.sparse_matrix(m, k, 0.8, 2, dist="normal", row_beta=True)
+    b = synth.dense_b(k, n, 3, dist="normal")
+    ref, _ = oracle.gemm_f32(a, b, n)
+    for split_k in (1, 6):
+        c, _, _ = run_spmm(product, a, b, n, split_k)
+        assert_close(c, ref, f"beta rows split_k={split_k}")

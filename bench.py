@@ -1,0 +1,193 @@
+#!/usr/bin/env python3
+"""Headline benchmark: one SpMM_SplitK_API call per step on one MI355X.
+
+Workload (BASELINE.json configs[2], the shape the metric is quoted on): the FFN up-projection
+A = 36864 x 9216 fp16 at 80 % unstructured sparsity, nonzeros ~ N(0, 0.02); B = 9216 x 16 fp16 ~ N(0,1).
+A step is the whole API call (SpMM kernel + split-K reduction) with Compressed_A, TileOffsets and B
+resident in HBM.  Steps rotate over several device copies of Compressed_A (272 MB each, more than the
+256 MB Infinity Cache together) so every launch streams its weights from HBM.
+
+Prints one JSON line; `value` = dense-equivalent TFLOPS = 2*M*N*K / t (the reference's formula,
+kernel_benchmark/spmm_test.cu:314-316).  `roofline` is for the SpMM kernel alone, timed live with
+events on the launch stream; `cpu_baseline` times the CPU oracle (compression on one thread, fp32 GEMM
+on all host cores) on the same workload and is a reported figure, not a target.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "flash-llm_amd"))
+
+HBM_PEAK_GBS = 8000.0
+
+# HBM bytes per SpMM-kernel launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# command, scaled by the same counters on a copy kernel of known size; None until measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def algorithmic_bytes(nnz_padded, m, n, k):
+    """Compressed_A + TileOffsets + B once + C once."""
+    return 4 * nnz_padded + 4 * ((m // 128) * (k // 64) + 2) + 2 * k * n + 2 * m * n
+
+
+def cpu_baseline(a, b, n):
+    """The reference's CPU path restated by the oracle: host compression (single thread, as the
+    reference) and an fp32 GEMM on the decompressed weights over all host cores."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import oracle
+
+    m, k = a.shape
+    t0 = time.perf_counter()
+    _, items, offsets = oracle.compress_reorder(a)
+    t_compress = time.perf_counter() - t0
+    dense = oracle.scatter(items, offsets, m, k)
+    best = None
+    threads = 1
+    for _ in range(3):
+        t0 = time.perf_counter()
+        _, threads = oracle.gemm_f32(dense, b, n)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    return {
+        "value": 2.0 * m * n * k / best / 1e12,
+        "unit": "TFLOPS",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"whole workload {m}x{k}x{n}: fp32 GEMM on decompressed weights, best of 3 on {threads} threads; "
+                  f"Tiled-CSL compression of the same matrix on 1 thread reported beside it",
+        "gemm_ms": best * 1e3,
+        "compress_s_1thread": t_compress,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--m", type=int, default=36864)
+    ap.add_argument("--k", type=int, default=9216)
+    ap.add_argument("--n", type=int, default=16)
+    ap.add_argument("--sparsity", type=float, default=0.8)
+    ap.add_argument("--split-k", type=int, default=0, help="0 = the library's heuristic")
+    ap.add_argument("--copies", type=int, default=4, help="device copies of Compressed_A to rotate over")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-dense", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (rows of A shard with no exchange; "
+                 "see DESIGN.md). Run with --gpus 1.")
+
+    import numpy as np
+    import torch
+
+    import flashllm_spmm as F
+    import synth
+
+    F.lib()  # fails loudly if libSpMM_API.so is not built
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    m, k, n = args.m, args.k, args.n
+    threads = min(16, os.cpu_count() or 1)
+    a = synth.sparse_matrix(m, k, args.sparsity, 0, dist="normal", sigma=0.02, threads=threads)
+    b_h = synth.dense_b(k, n, 0, dist="normal")
+    items, offsets = F.init_sparse_matrix_a(a)
+    nnz = int(items.size)
+    split_k = args.split_k or F.splitk_heuristic(m, n, k)
+
+    dev = "cuda"
+    comps = [torch.from_numpy(items.view(np.int32)).to(dev) for _ in range(max(1, args.copies))]
+    offs = torch.from_numpy(offsets).to(dev)
+    b = torch.from_numpy(b_h).to(dev)
+    c = torch.empty(n * m, dtype=torch.float16, device=dev)
+    ws = torch.empty(max(1, split_k) * n * m, dtype=torch.float16, device=dev)
+
+    def step(i):
+        F.spmm_splitk(comps[i % len(comps)], offs, b, c, m, n, k, ws, split_k)
+
+    def kernel_only(i):
+        F.spmm_partials(comps[i % len(comps)], offs, b, c, m, n, k, ws, split_k)
+
+    def timed(fn, steps, warmup):
+        for i in range(warmup):
+            fn(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(steps):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps  # ms per call
+
+    ms_step = timed(step, args.steps, args.warmup)
+    ms_kernel = timed(kernel_only, args.steps, args.warmup)
+
+    # correctness of what was just timed (cheap sample of rows against an fp32 product)
+    step(0)
+    torch.cuda.synchronize()
+    rows = np.arange(0, m, max(1, m // 512))
+    ref = b_h.astype(np.float32) @ a[rows].astype(np.float32).T
+    got = c.cpu().numpy().reshape(n, m)[:, rows].astype(np.float32)
+    rel_err = float(np.max(np.abs(got - ref)) / np.max(np.abs(ref)))
+
+    alg = algorithmic_bytes(nnz, m, n, k)
+    flops = 2.0 * m * n * k
+    achieved = alg / (ms_kernel * 1e-3) / 1e9
+    out = {
+        "metric": "dense-equiv TFLOPS + % HBM roofline, M=36864 K=9216 N=16, 80% sparse fp16",
+        "value": flops / (ms_step * 1e-3) / 1e12,
+        "unit": "TFLOPS",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"SpMM_SplitK_API {m}x{k} (80% sparse ffn up-projection) x {k}x{n}, Tiled-CSL, fp16 in / fp32 accumulate",
+            "M": m, "K": k, "N": n, "sparsity": args.sparsity, "split_k": split_k,
+            "nnz_padded": nnz, "compressed_a_copies_rotated": len(comps),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((m, k, n)),
+            "kernel": "spmm_stream_kernel",
+            "kernel_ms": ms_kernel,
+            "algorithmic_bytes": alg,
+        },
+        "whole_call": {
+            "effective_GBps": alg / (ms_step * 1e-3) / 1e9,
+            "frac_of_hbm_peak": alg / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "reduction_ms": max(ms_step - ms_kernel, 0.0),
+        },
+        "max_rel_err_sampled_rows": rel_err,
+    }
+
+    if not args.no_dense:
+        # dense fp16 GEMM of the same shape through the BLAS library torch ships (hipBLASLt/rocBLAS)
+        a_d = torch.from_numpy(a).to(dev)
+        bt = b.view(n, k).t().contiguous()  # K x N
+        ms_dense = timed(lambda i: torch.matmul(a_d, bt), max(10, args.steps // 4), 5)
+        out["dense_fp16_gemm"] = {"ms": ms_dense, "tflops": flops / (ms_dense * 1e-3) / 1e12,
+                                  "speedup_of_spmm": ms_dense / ms_step}
+        del a_d
+
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(a, b_h, n)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

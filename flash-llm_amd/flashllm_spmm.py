@@ -45,6 +45,13 @@ def lib():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise OSError(f"{LIB_PATH} is not built: run `make -C {_HERE}` (or __graft_entry__.build())")
+        # One HIP runtime per process: torch ships its own libamdhip64.so.7.  Loading it first makes
+        # the dynamic loader resolve this library's libamdhip64.so.7 dependency to that same copy;
+        # a second runtime in the process reports hipErrorNoDevice on its first launch.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         handle = ctypes.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(handle, name)

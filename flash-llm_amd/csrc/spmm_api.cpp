@@ -87,28 +87,35 @@ size_t flashllm_workspace_bytes(int m, int n, int split_k)
     return static_cast<size_t>(split_k) * m * n * sizeof(uint16_t);
 }
 
-// One wave streams one (row tile, K slice, column group) and owns 16 KB of
-// LDS, so a CU holds about eight of them; the grid should put roughly that
-// many on each of the 256 CUs, in slices of equal length.
+// One wave streams one (row tile, K slice, column group) and owns 16 KB of LDS for its tile plus
+// 4 KB per 16 output columns for B staging, so a CU (160 KB) holds 8 / 6 / 5 of them for
+// N <= 16 / 32 / >= 64.  The grid should fill those slots on all 256 CUs exactly once, in slices of
+// equal length: a second round of workgroups would run at a fraction of the occupancy.
 int flashllm_splitk_heuristic(int m, int n, int k)
 {
     if (m <= 0 || k <= 0 || n <= 0 || m % 128 || k % 64)
         return 1;
     const int  kt         = k / 64;
+    const int  nb         = n <= 16 ? 1 : (n == 32 ? 2 : 4);
     const int  col_groups = n <= 64 ? 1 : n / 64;
     const long units      = static_cast<long>(m / 128) * col_groups;
-    const long target     = 256L * 8;
-    int        best       = 1;
-    double     best_cost  = 1e30;
-    for (int s = 1; s <= kt && s <= 32; s++) {
-        const int  avg   = (kt - 1) / s + 1;  // longest slice, in k tiles
-        const long waves = units * s;
-        // time ~ rounds of resident waves x longest slice, plus slab traffic
-        const long   rounds = (waves + target - 1) / target;
-        const double stream = static_cast<double>(rounds) * avg;
-        const double slabs  = s > 1 ? 0.04 * s * kt / 8.0 : 0.0;
-        const double idle   = waves < target ? static_cast<double>(target - waves) / target * avg * 0.5 : 0.0;
-        const double cost   = stream + slabs + idle;
+    const long slots      = 256L * (160 / (16 + 4 * nb));
+    // Largest split that still runs in one round; a second round would run at a fraction of the
+    // occupancy (measured at 36864x9216, N=16: 51 us at 7 slices = 2016 waves, 70 us at 8).
+    long s_max = slots / units;
+    if (s_max > 32)
+        s_max = 32;  // workspace sizes in existing callers assume at most 32 slabs
+    if (s_max > kt)
+        s_max = kt;
+    if (s_max < 1)
+        s_max = 1;
+    // Time follows the longest slice (in k tiles); each slab adds a write and a read of M*N halfs
+    // and a little reduction time, about a quarter of a k tile's worth.
+    int    best      = 1;
+    double best_cost = 1e30;
+    for (int s = 1; s <= s_max; s++) {
+        const int    avg  = (kt - 1) / s + 1;
+        const double cost = avg + (s > 1 ? 0.25 * s : 0.0);
         if (cost < best_cost) {
             best_cost = cost;
             best      = s;

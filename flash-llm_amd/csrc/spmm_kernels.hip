@@ -7,19 +7,28 @@
 //   * A wave owns one 128-row tile row of A, one K slice and one group of
 //     output columns.  The slice's packed nonzeros are one contiguous range
 //     of Compressed_A (tiles of a tile row are stored back to back), so the
-//     wave streams it as 1 KB chunks (64 lanes x 16 B, coalesced, aligned)
-//     through a ring of DEPTH register slots that is always DEPTH chunks
-//     ahead, whatever the tile boundaries are.
+//     wave streams it as 1 KB chunks (64 lanes x 16 B, coalesced, aligned,
+//     non-temporal) through a ring of DEPTH register slots that stays DEPTH
+//     chunks ahead, whatever the tile boundaries are.
 //   * Each chunk is scattered into the wave's private 128x64 fp16 tile in LDS
 //     at the position stored in the item (the format's XOR-swizzled layout,
 //     reference csrc/SpMM_API.cu:252-261).  When the running vector index
 //     passes TileOffsets[t+1] the tile is complete: the wave reads it back as
 //     16 ds_read_b128 MFMA operands (the swizzle makes every group of eight
-//     lanes hit 32 distinct banks), issues v_mfma_f32_16x16x32_f16 against B
-//     fragments taken straight from global/L2 (column-major B already is the
-//     MFMA operand layout: 8 consecutive k per lane), and clears the tile.
-//   * One wave, in-order LDS: no barrier anywhere.  Any tile density works,
-//     empty tiles and empty slices included.
+//     lanes hit 32 distinct banks), issues v_mfma_f32_16x16x32_f16 against the
+//     B fragments of that k tile (column-major B already is the MFMA operand
+//     layout: 8 consecutive k per lane), and clears the tile.  Any number of
+//     tiles may end inside one chunk (empty tiles, tiles of a single vector).
+//   * One wave, in-order LDS: no barrier anywhere.
+//
+// Waiting for memory.  The ring loads are the only vector-memory loads the
+// compiler sees, and every path through a ring stage issues exactly one, so
+// its wait before a slot is used is the exact vmcnt(DEPTH-1).  The B fragments
+// of the next tile travel global -> LDS with global_load_lds_dwordx4 issued
+// from inline assembly when the tile is opened, and are awaited when it
+// completes with an explicit vmcnt derived from the number of ring loads
+// issued in between.  The compiler does not know about these loads; extra
+// loads in flight only make its own vmcnt waits stricter, never weaker.
 //
 // splitk_reduce_kernel: the separate reduction over fp16 slabs
 // (reference csrc/Reduction_Kernel.cuh:24-45), 16 bytes per lane per slab.
@@ -33,11 +42,13 @@ namespace {
 using half8   = _Float16 __attribute__((ext_vector_type(8)));
 using half4   = _Float16 __attribute__((ext_vector_type(4)));
 using floatx4 = float __attribute__((ext_vector_type(4)));
+using uintx4  = uint32_t __attribute__((ext_vector_type(4)));
 
 constexpr int kTileRows  = 128;
 constexpr int kTileCols  = 64;
 constexpr int kTileHalfs = kTileRows * kTileCols;
 constexpr int kLanes     = 64;
+constexpr int kNoTile    = 0x7fffffff;
 
 __device__ __forceinline__ void clear_tile(uint16_t* tile, int lane)
 {
@@ -54,7 +65,51 @@ __device__ __forceinline__ void scatter_item(uint16_t* tile, uint32_t item)
     tile[(item >> 16) & (kTileHalfs - 1)] = static_cast<uint16_t>(item);
 }
 
-template<int NB, int DEPTH>
+__device__ __forceinline__ void scatter_vector(uint16_t* tile, const uint4& v)
+{
+    scatter_item(tile, v.x);
+    scatter_item(tile, v.y);
+    scatter_item(tile, v.z);
+    scatter_item(tile, v.w);
+}
+
+// streaming load of one 16-byte vector: the weights are read once, keep them out of the caches' way
+__device__ __forceinline__ uint4 load_stream(const uint4* p)
+{
+    const uintx4 x = __builtin_nontemporal_load(reinterpret_cast<const uintx4*>(p));
+    return uint4{x[0], x[1], x[2], x[3]};
+}
+
+__device__ __forceinline__ uint32_t lds_offset(const void* p)
+{
+    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) void*)(p)));
+}
+
+// 16 bytes per lane, global -> LDS at lds_byte_addr + lane*16, without passing through registers.
+// Counted by vmcnt like any load, but invisible to the compiler's wait insertion.
+__device__ __forceinline__ void load_to_lds_16(const void* g, uint32_t lds_byte_addr)
+{
+    uint32_t saved;
+    asm volatile("s_mov_b32 %0, m0\n\t"
+                 "s_mov_b32 m0, %2\n\t"
+                 "s_nop 0\n\t"
+                 "global_load_lds_dwordx4 %1, off\n\t"
+                 "s_mov_b32 m0, %0\n\t"
+                 : "=&s"(saved)
+                 : "v"(g), "s"(lds_byte_addr)
+                 : "memory");
+}
+
+template<int W>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(W) : "memory");
+}
+
+// NB: 16-column blocks per wave (1 for N <= 16, 2 for N = 32, 4 for N >= 64).
+// DEPTH: ring slots = 1 KB chunks in flight per wave.
+// BWAIT: a B request followed by at least BWAIT ring loads is awaited with vmcnt(BWAIT).
+template<int NB, int DEPTH, int BWAIT>
 __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __restrict__ comp,
                                                             const int* __restrict__ offs,
                                                             const _Float16* __restrict__ B,
@@ -65,6 +120,7 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                                                             int split_k)
 {
     __shared__ __attribute__((aligned(16))) uint16_t tile[kTileHalfs];
+    __shared__ __attribute__((aligned(16))) uint32_t bstage[2][2 * NB][256];  // [tile parity][k step, block][lane*4]
 
     const int lane    = threadIdx.x;
     const int r16     = lane & 15;  // row inside a 16-row block / output column
@@ -99,10 +155,19 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
         const _Float16* bptr[NB];
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) {
-            int n = col0 + nb * 16 + r16;
-            n     = n < N ? n : N - 1;  // N == 8: lanes 8..15 compute columns nobody stores
+            int n    = col0 + nb * 16 + r16;
+            n        = n < N ? n : N - 1;  // N == 8: lanes 8..15 compute columns nobody stores
             bptr[nb] = B + static_cast<size_t>(n) * K + g * 8;
         }
+        const uint32_t bstage_lds = lds_offset(&bstage[0][0][0]);
+        auto           request_b  = [&](int t) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                for (int nb = 0; nb < NB; nb++)
+                    load_to_lds_16(bptr[nb] + t * kTileCols + ks * 32,
+                                   bstage_lds + (((t & 1) * 2 * NB + ks * NB + nb) << 10));
+        };
 
         clear_tile(tile, lane);
 
@@ -111,80 +176,77 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
         const int vlast   = vend - 1;
         uint4     ring[DEPTH];
 #pragma unroll
-        for (int d = 0; d < DEPTH; d++) {
-            int v   = cbase + d * kLanes + lane;
-            v       = v < vlast ? v : vlast;
-            ring[d] = comp[v];
-        }
+        for (int d = 0; d < DEPTH; d++)
+            ring[d] = uint4{0u, 0u, 0u, 0u};
 
-        int   t       = kb;
-        int   tile_lo = vbeg;
-        int   tile_hi = toff[t + 1];
-        half8 bfrag[2][NB];
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-            bfrag[0][nb] = *reinterpret_cast<const half8*>(bptr[nb] + t * kTileCols);
-            bfrag[1][nb] = *reinterpret_cast<const half8*>(bptr[nb] + t * kTileCols + 32);
-        }
+        int t = kb, tile_lo = vbeg, tile_hi = toff[kb + 1], next_hi = toff[kb + 2];
+        int since = 0;  // ring loads issued after the latest B request
+        request_b(t);
 
-        bool done = false;
-        for (int c0 = 0; c0 < nchunks && !done; c0 += DEPTH) {
+        // Chunks -DEPTH .. -1 only fill the ring: none of their lanes reaches tile_lo, and a tile can
+        // only "end" there when it is empty.
+        for (int c0 = -DEPTH; c0 < nchunks; c0 += DEPTH) {
 #pragma unroll
             for (int d = 0; d < DEPTH; d++) {
-                const int c = c0 + d;
-                if (c >= nchunks || done)
-                    break;
-                const uint4 cur = ring[d];
+                const int v  = cbase + (c0 + d) * kLanes + lane;  // this lane's vector
+                const int ve = cbase + (c0 + d + 1) * kLanes;     // end of the chunk
                 {
-                    int v   = cbase + (c + DEPTH) * kLanes + lane;
-                    v       = v < vlast ? v : vlast;
-                    ring[d] = comp[v];
-                }
-                const int vb = cbase + c * kLanes;
-                const int v  = vb + lane;
-                for (;;) {
-                    const int hi = tile_hi < vb + kLanes ? tile_hi : vb + kLanes;
-                    if (v >= tile_lo && v < hi) {
-                        scatter_item(tile, cur.x);
-                        scatter_item(tile, cur.y);
-                        scatter_item(tile, cur.z);
-                        scatter_item(tile, cur.w);
-                    }
-                    if (tile_hi > vb + kLanes)
-                        break;  // the tile continues in the next chunk
-                    if (tile_hi > tile_lo) {
-                        const char* base = reinterpret_cast<const char*>(tile);
+                    const uint4 cur = ring[d];
+                    if (v >= tile_lo && v < tile_hi)
+                        scatter_vector(tile, cur);
+                    while (tile_hi <= ve) {  // a tile ends inside, or exactly at the end of, this chunk
+                        if (tile_hi > tile_lo) {
+                            if (since >= BWAIT)
+                                wait_vmcnt<BWAIT>();
+                            else
+                                wait_vmcnt<0>();
+                            const char*  base = reinterpret_cast<const char*>(tile);
+                            const uint4* bs   = reinterpret_cast<const uint4*>(&bstage[t & 1][0][0]);
 #pragma unroll
-                        for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-                            for (int rb = 0; rb < 8; rb++) {
-                                const half8 a = *reinterpret_cast<const half8*>(
-                                    base + rb * (16 * kTileCols * 2) + (ks ? a_off1 : a_off0));
+                            for (int ks = 0; ks < 2; ks++) {
+                                half8 bfrag[NB];
 #pragma unroll
                                 for (int nb = 0; nb < NB; nb++)
-                                    acc[nb][rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                        a, bfrag[ks][nb], acc[nb][rb], 0, 0, 0);
-                            }
-                        clear_tile(tile, lane);
-                    }
-                    t++;
-                    if (t >= ke) {
-                        done = true;
-                        break;
-                    }
+                                    bfrag[nb] = __builtin_bit_cast(half8, bs[(ks * NB + nb) * kLanes + lane]);
 #pragma unroll
-                    for (int nb = 0; nb < NB; nb++) {
-                        bfrag[0][nb] = *reinterpret_cast<const half8*>(bptr[nb] + t * kTileCols);
-                        bfrag[1][nb] = *reinterpret_cast<const half8*>(bptr[nb] + t * kTileCols + 32);
+                                for (int rb = 0; rb < 8; rb++) {
+                                    const half8 a = *reinterpret_cast<const half8*>(
+                                        base + rb * (16 * kTileCols * 2) + (ks ? a_off1 : a_off0));
+#pragma unroll
+                                    for (int nb = 0; nb < NB; nb++)
+                                        acc[nb][rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                            a, bfrag[nb], acc[nb][rb], 0, 0, 0);
+                                }
+                            }
+                            clear_tile(tile, lane);
+                        }
+                        t++;
+                        tile_lo = tile_hi;
+                        if (t < ke) {
+                            request_b(t);
+                            since   = 0;
+                            tile_hi = next_hi;
+                            next_hi = toff[t + 2];
+                            if (v >= tile_lo && v < tile_hi)  // the rest of this chunk opens the next tile
+                                scatter_vector(tile, cur);
+                        }
+                        else {  // nothing left: the remaining stages are no-ops
+                            tile_lo = kNoTile;
+                            tile_hi = kNoTile;
+                        }
                     }
-                    tile_lo = tile_hi;
-                    tile_hi = toff[t + 1];
+                }
+                {
+                    int vn  = v + DEPTH * kLanes;
+                    vn      = vn < vlast ? vn : vlast;
+                    ring[d] = load_stream(comp + vn);
+                    since++;
                 }
             }
         }
     }
 
-    // D layout of the 16x16 MFMA: lane holds column r16, rows 4*g .. 4*g+3.
+    // D layout of the 16x16 MFMA: lane holds column r16, rows 4*g .. 4*g+3 of each 16-row block.
     _Float16* o = out + static_cast<size_t>(slice) * M * N + static_cast<size_t>(rowtile) * kTileRows + g * 4;
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) {
@@ -240,11 +302,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(uint4* __restrict__ 
     c[i] = __builtin_bit_cast(uint4, h);
 }
 
-template<int NB, int DEPTH>
+template<int NB, int DEPTH, int BWAIT>
 int launch_spmm(hipStream_t stream, const void* comp, const int* offs, const void* b, void* out, int m, int n, int k, int split_k, int col_groups)
 {
     const dim3 grid(static_cast<unsigned>(m / kTileRows) * split_k, col_groups, 1);
-    hipLaunchKernelGGL((spmm_stream_kernel<NB, DEPTH>),
+    hipLaunchKernelGGL((spmm_stream_kernel<NB, DEPTH, BWAIT>),
                        grid,
                        dim3(kLanes),
                        0,
@@ -267,10 +329,10 @@ extern "C" int flashllm_hip_launch_spmm(
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (n <= 16)
-        return launch_spmm<1, 8>(s, comp, offs, b, out, m, n, k, split_k, 1);
+        return launch_spmm<1, 8, 4>(s, comp, offs, b, out, m, n, k, split_k, 1);
     if (n == 32)
-        return launch_spmm<2, 8>(s, comp, offs, b, out, m, n, k, split_k, 1);
-    return launch_spmm<4, 8>(s, comp, offs, b, out, m, n, k, split_k, n / 64);
+        return launch_spmm<2, 8, 4>(s, comp, offs, b, out, m, n, k, split_k, 1);
+    return launch_spmm<4, 8, 4>(s, comp, offs, b, out, m, n, k, split_k, n / 64);
 }
 
 extern "C" int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws, long mn, int split_k)

@@ -23,9 +23,11 @@ sys.path.insert(0, os.path.join(ROOT, "flash-llm_amd"))
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per SpMM-kernel launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# command, scaled by the same counters on a copy kernel of known size; None until measured.
-MEASURED_TRAFFIC_BYTES = {}
+# HBM bytes per SpMM-kernel launch at the default Split_K, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs of this command, each scaled by what the same counter reads for the 256 MiB copy of
+# --calibrate-copy (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); profiles/ holds the summary.  Shapes that
+# were not profiled report null.
+MEASURED_TRAFFIC_BYTES = {(36864, 9216, 16, 7): 284849874}
 
 
 def algorithmic_bytes(nnz_padded, m, n, k):
@@ -75,6 +77,9 @@ def main():
     ap.add_argument("--split-k", type=int, default=0, help="0 = the library's heuristic")
     ap.add_argument("--copies", type=int, default=4, help="device copies of Compressed_A to rotate over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain device-to-device copy of 256 MiB: the known-size kernel the FETCH_SIZE / "
+                         "WRITE_SIZE counters are scaled by")
     ap.add_argument("--no-dense", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -160,7 +165,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((m, k, n)),
+            "traffic": MEASURED_TRAFFIC_BYTES.get((m, k, n, split_k)) if abs(args.sparsity - 0.8) < 1e-9 else None,
             "kernel": "spmm_stream_kernel",
             "kernel_ms": ms_kernel,
             "algorithmic_bytes": alg,
@@ -172,6 +177,13 @@ def main():
         },
         "max_rel_err_sampled_rows": rel_err,
     }
+
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        ms_copy = timed(lambda i: dst.copy_(src), 10, 2)
+        out["copy_256MiB"] = {"ms": ms_copy, "GBps_read_plus_write": 2 * (256 << 20) / (ms_copy * 1e-3) / 1e9}
+        del src, dst
 
     if not args.no_dense:
         # dense fp16 GEMM of the same shape through the BLAS library torch ships (hipBLASLt/rocBLAS)

@@ -16,7 +16,8 @@ extern "C" {
 /* Error codes of the host-side functions (negative return values). */
 #define FLASHLLM_E_SHAPE (-1)   /* M % 128 != 0, K % 64 != 0 or not positive */
 #define FLASHLLM_E_NOMEM (-2)   /* host allocation failed */
-#define FLASHLLM_E_NOZERO (-3)  /* padding needed in a bank with no zero position */
+#define FLASHLLM_E_NOZERO (-3)  /* padding needed in a bank with no zero position (the reference asserts; unreachable:
+                                   the emptiest bank always has one) */
 #define FLASHLLM_E_ARG (-5)     /* null pointer */
 #define FLASHLLM_E_IO (-6)      /* file could not be opened / short read */
 

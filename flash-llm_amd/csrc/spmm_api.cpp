@@ -57,7 +57,7 @@ int flashllm_spmm_partials(void*       stream,
 
 int flashllm_splitk_reduce(void* stream, void* c, const void* ws, int m, int n, int split_k)
 {
-    if (!c || !ws || m <= 0 || n <= 0 || split_k < 1 || (static_cast<long>(m) * n) % 8)
+    if (!c || !ws || m <= 0 || n <= 0 || split_k < 1 || (static_cast<long>(m) * n) % 4)
         return hipErrorInvalidValue;
     return flashllm_hip_launch_reduce(stream, c, ws, static_cast<long>(m) * n, split_k);
 }
@@ -88,8 +88,8 @@ size_t flashllm_workspace_bytes(int m, int n, int split_k)
 }
 
 // One wave streams one (row tile, K slice, column group) and owns 16 KB of LDS for its tile plus
-// 4 KB per 16 output columns for B staging, so a CU (160 KB) holds 8 / 6 / 5 of them for
-// N <= 16 / 32 / >= 64.  The grid should fill those slots on all 256 CUs exactly once, in slices of
+// 4 KB per 16 output columns for B staging, so a CU (160 KB) holds 8 / 6 / 4 of them for
+// N <= 16 / 32 / >= 64 (five 32 KB workgroups would need all 160 KB; only four become resident).  The grid should fill those slots on all 256 CUs exactly once, in slices of
 // equal length: a second round of workgroups would run at a fraction of the occupancy.
 int flashllm_splitk_heuristic(int m, int n, int k)
 {
@@ -99,7 +99,7 @@ int flashllm_splitk_heuristic(int m, int n, int k)
     const int  nb         = n <= 16 ? 1 : (n == 32 ? 2 : 4);
     const int  col_groups = n <= 64 ? 1 : n / 64;
     const long units      = static_cast<long>(m / 128) * col_groups;
-    const long slots      = 256L * (160 / (16 + 4 * nb));
+    const long slots      = 256L * (nb == 4 ? 4 : 160 / (16 + 4 * nb));
     // Largest split that still runs in one round; a second round would run at a fraction of the
     // occupancy (measured at 36864x9216, N=16: 51 us at 7 slices = 2016 waves, 70 us at 8).
     long s_max = slots / units;
@@ -122,6 +122,55 @@ int flashllm_splitk_heuristic(int m, int n, int k)
         }
     }
     return best;
+}
+
+// The four pruned linears of a decoder layer, in the order and with the Split_K fallbacks of the
+// reference's FasterTransformer call sites (third_party/ft.patch:512-525, :615-633, :1247-1261,
+// :1328-1340, :1444-1456, :1508-1521).
+int flashllm_decoder_layer_linears(void*                         stream,
+                                   const flashllm_decoder_layer* layer,
+                                   const void*                   x,
+                                   void*                         qkv_out,
+                                   void*                         attn_in,
+                                   void*                         attn_out,
+                                   void*                         ffn_mid,
+                                   void*                         y,
+                                   int                           tokens,
+                                   void*                         ws)
+{
+    if (!layer || !x || !qkv_out || !attn_in || !attn_out || !ffn_mid || !y)
+        return hipErrorInvalidValue;
+    const flashllm_sparse_weight& q = layer->qkv;
+    const flashllm_sparse_weight& o = layer->attn_out;
+    const flashllm_sparse_weight& f1 = layer->ffn1;
+    const flashllm_sparse_weight& f2 = layer->ffn2;
+    const int hidden = q.k;
+    if (o.k != hidden || q.m < hidden || f1.k != o.m || f2.k != f1.m || hidden % 8 || q.m % 8)
+        return hipErrorInvalidValue;
+    auto split = [&](const flashllm_sparse_weight& w, int limit) {
+        if (tokens > limit)
+            return 1;
+        return w.split_k > 0 ? w.split_k : flashllm_splitk_heuristic(w.m, tokens, w.k);
+    };
+    auto linear = [&](const flashllm_sparse_weight& w, const void* in, void* out, int limit) {
+        return flashllm_spmm_splitk(stream, nullptr, w.nz_weights, w.tile_offsets, in, out, w.m, tokens, w.k, ws, split(w, limit));
+    };
+    int rc = linear(q, x, qkv_out, 64);
+    if (rc)
+        return rc;
+    rc = flashllm_hip_launch_take_rows(stream, attn_in, qkv_out, hidden, tokens, q.m);
+    if (rc)
+        return rc;
+    rc = linear(o, attn_in, attn_out, 64);
+    if (rc)
+        return rc;
+    rc = linear(f1, attn_out, ffn_mid, 128);
+    if (rc)
+        return rc;
+    rc = flashllm_hip_launch_relu(stream, ffn_mid, static_cast<long>(f1.m) * tokens);
+    if (rc)
+        return rc;
+    return linear(f2, ffn_mid, y, 128);
 }
 
 }  // extern "C"

@@ -31,7 +31,7 @@
 // loads in flight only make its own vmcnt waits stricter, never weaker.
 //
 // splitk_reduce_kernel: the separate reduction over fp16 slabs
-// (reference csrc/Reduction_Kernel.cuh:24-45), 16 bytes per lane per slab.
+// (reference csrc/Reduction_Kernel.cuh:24-45), 8 bytes per lane per slab, eight slabs in flight.
 #include "spmm_launch.h"
 
 #include <hip/hip_runtime.h>
@@ -129,6 +129,8 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
     const int slice   = blockIdx.x % split_k;
     const int rowtile = blockIdx.x / split_k;
     const int col0    = blockIdx.y * (16 * NB);
+    // HW_ID.wave_id: which of the SIMD's wave slots this wave sits in (bit 0 tells the two apart)
+    const int wave_slot = __builtin_amdgcn_s_getreg(4 | (0 << 6) | (3 << 11)) & 1;
 
     // the reference's slicing (csrc/SpMM_Kernel.cuh:196-204), clamped to K
     const int avg = (kt - 1) / split_k + 1;
@@ -222,6 +224,13 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                         }
                         t++;
                         tile_lo = tile_hi;
+                        // The SIMD's arbiter serves its older wave first, which leaves the younger of the two
+                        // resident waves about 17 % slower; taking turns at raised priority, one tile each,
+                        // evens their finishing times.
+                        if ((t ^ wave_slot) & 1)
+                            __builtin_amdgcn_s_setprio(1);
+                        else
+                            __builtin_amdgcn_s_setprio(0);
                         if (t < ke) {
                             request_b(t);
                             since   = 0;
@@ -265,41 +274,84 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
     }
 }
 
-__device__ __forceinline__ void add_slab(float (&s)[8], const uint4 v)
+__device__ __forceinline__ void add_slab(float (&s)[4], const uint2 v)
 {
-    const half8 h = __builtin_bit_cast(half8, v);
+    const half4 h = __builtin_bit_cast(half4, v);
 #pragma unroll
-    for (int j = 0; j < 8; j++)
+    for (int j = 0; j < 4; j++)
         s[j] += static_cast<float>(h[j]);
 }
 
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(uint4* __restrict__ c,
-                                                           const uint4* __restrict__ ws,
-                                                           long n8,
+// C[e] = rn16(sum over slabs, in slab order, of float(ws[s*MN + e])).  Eight bytes per lane and up to
+// eight slabs in flight per lane: the slabs are small (M*N halfs), so the kernel is latency bound and
+// wants many independent loads rather than wide ones.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(uint2* __restrict__ c,
+                                                           const uint2* __restrict__ ws,
+                                                           long n4,
                                                            int  split_k)
+{
+    const long i = static_cast<long>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= n4)
+        return;
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    int   k    = 0;
+    for (; k + 8 <= split_k; k += 8) {
+        uint2 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            v[j] = ws[(k + j) * n4 + i];
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            add_slab(s, v[j]);
+    }
+    if (k + 4 <= split_k) {
+        uint2 v[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            v[j] = ws[(k + j) * n4 + i];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            add_slab(s, v[j]);
+        k += 4;
+    }
+    {
+        uint2 v[3];
+        const int left = split_k - k;  // 0..3
+#pragma unroll
+        for (int j = 0; j < 3; j++)
+            if (j < left)
+                v[j] = ws[(k + j) * n4 + i];
+#pragma unroll
+        for (int j = 0; j < 3; j++)
+            if (j < left)
+                add_slab(s, v[j]);
+    }
+    half4 h;
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        h[j] = static_cast<_Float16>(s[j]);
+    c[i] = __builtin_bit_cast(uint2, h);
+}
+
+__global__ __launch_bounds__(256) void relu_kernel(uint4* __restrict__ x, long n8)
 {
     const long i = static_cast<long>(blockIdx.x) * 256 + threadIdx.x;
     if (i >= n8)
         return;
-    float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    int   k    = 0;
-    for (; k + 4 <= split_k; k += 4) {
-        const uint4 v0 = ws[(k + 0) * n8 + i];
-        const uint4 v1 = ws[(k + 1) * n8 + i];
-        const uint4 v2 = ws[(k + 2) * n8 + i];
-        const uint4 v3 = ws[(k + 3) * n8 + i];
-        add_slab(s, v0);
-        add_slab(s, v1);
-        add_slab(s, v2);
-        add_slab(s, v3);
-    }
-    for (; k < split_k; k++)
-        add_slab(s, ws[k * n8 + i]);
-    half8 h;
+    half8 h = __builtin_bit_cast(half8, x[i]);
 #pragma unroll
     for (int j = 0; j < 8; j++)
-        h[j] = static_cast<_Float16>(s[j]);
-    c[i] = __builtin_bit_cast(uint4, h);
+        h[j] = h[j] > static_cast<_Float16>(0) ? h[j] : static_cast<_Float16>(0);  // NaN -> 0 like max(x, 0)
+    x[i] = __builtin_bit_cast(uint4, h);
+}
+
+__global__ __launch_bounds__(256) void take_rows_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, int rows8, int cols, int ld8)
+{
+    const long i = static_cast<long>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= static_cast<long>(rows8) * cols)
+        return;
+    const int j = static_cast<int>(i / rows8), r = static_cast<int>(i % rows8);
+    dst[i] = src[static_cast<long>(j) * ld8 + r];
 }
 
 template<int NB, int DEPTH, int BWAIT>
@@ -337,15 +389,32 @@ extern "C" int flashllm_hip_launch_spmm(
 
 extern "C" int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws, long mn, int split_k)
 {
-    const long n8 = mn / 8;
+    const long n4 = mn / 4;
     hipLaunchKernelGGL(splitk_reduce_kernel,
-                       dim3(static_cast<unsigned>((n8 + 255) / 256)),
+                       dim3(static_cast<unsigned>((n4 + 255) / 256)),
                        dim3(256),
                        0,
                        static_cast<hipStream_t>(stream),
-                       static_cast<uint4*>(c),
-                       static_cast<const uint4*>(ws),
-                       n8,
+                       static_cast<uint2*>(c),
+                       static_cast<const uint2*>(ws),
+                       n4,
                        split_k);
+    return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int flashllm_hip_launch_relu(void* stream, void* x, long n)
+{
+    const long n8 = n / 8;
+    hipLaunchKernelGGL(relu_kernel, dim3(static_cast<unsigned>((n8 + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<uint4*>(x), n8);
+    return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int flashllm_hip_launch_take_rows(void* stream, void* dst, const void* src, int rows, int cols, int src_ld)
+{
+    const long n8 = static_cast<long>(rows / 8) * cols;
+    hipLaunchKernelGGL(take_rows_kernel, dim3(static_cast<unsigned>((n8 + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<uint4*>(dst), static_cast<const uint4*>(src),
+                       rows / 8, cols, src_ld / 8);
     return static_cast<int>(hipGetLastError());
 }

@@ -20,8 +20,14 @@ int flashllm_hip_launch_spmm(void*       stream,
                              int         k,
                              int         split_k);
 
-// c[e] = rn16(sum_s float(ws[s*mn + e])); requires mn % 8 == 0.
+// c[e] = rn16(sum_s float(ws[s*mn + e])); requires mn % 4 == 0.
 int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws, long mn, int split_k);
+
+// x[i] = max(x[i], 0) over n halfs (n % 8 == 0): the activation between FFN1 and FFN2.
+int flashllm_hip_launch_relu(void* stream, void* x, long n);
+
+// dst[j*rows + i] = src[j*src_ld + i] for i < rows, j < cols (rows % 8 == 0, src_ld % 8 == 0).
+int flashllm_hip_launch_take_rows(void* stream, void* dst, const void* src, int rows, int cols, int src_ld);
 
 #ifdef __cplusplus
 }

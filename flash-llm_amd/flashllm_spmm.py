@@ -23,6 +23,18 @@ _u32p = ctypes.POINTER(ctypes.c_uint32)
 _i32p = ctypes.POINTER(ctypes.c_int)
 _vp = ctypes.c_void_p
 
+class SparseWeightStruct(ctypes.Structure):
+    """flashllm_sparse_weight"""
+    _fields_ = [("nz_weights", ctypes.c_void_p), ("tile_offsets", ctypes.c_void_p),
+                ("m", ctypes.c_int), ("k", ctypes.c_int), ("split_k", ctypes.c_int)]
+
+
+class DecoderLayerStruct(ctypes.Structure):
+    """flashllm_decoder_layer"""
+    _fields_ = [("qkv", SparseWeightStruct), ("attn_out", SparseWeightStruct),
+                ("ffn1", SparseWeightStruct), ("ffn2", SparseWeightStruct)]
+
+
 # name -> (restype, argtypes); every symbol include/flashllm_spmm.h declares
 SIGNATURES = {
     "flashllm_init_sparse_matrix_a": (ctypes.c_int, [_u16p, ctypes.c_int, ctypes.c_int, ctypes.POINTER(_u32p), ctypes.POINTER(_i32p)]),
@@ -34,6 +46,7 @@ SIGNATURES = {
     "flashllm_splitk_reduce": (ctypes.c_int, [_vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "flashllm_splitk_heuristic": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "flashllm_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "flashllm_decoder_layer_linears": (ctypes.c_int, [_vp, ctypes.POINTER(DecoderLayerStruct), _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp]),
     "flashllm_gen_sparse_matrix_bin_file": (ctypes.c_int, [ctypes.c_char_p, ctypes.c_int, ctypes.c_int, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_char_p]),
     "GenSparseMatrixBinFile": (None, [ctypes.c_char_p, ctypes.c_int, ctypes.c_int, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_char_p]),
 }
@@ -185,3 +198,37 @@ class SparseWeight:
             workspace = torch.empty(s * n * self.m, dtype=torch.float16, device=self.device)
         spmm_splitk(self.comp, self.offs, b, c, self.m, n, self.k, workspace, s, stream=stream)
         return c
+
+    def as_struct(self):
+        return SparseWeightStruct(self.comp.data_ptr(), self.offs.data_ptr(), self.m, self.k, self.split_k or 0)
+
+
+class DecoderLayer:
+    """The four pruned linears of one decoder layer (QKV, attention output, FFN1, FFN2) on the GPU."""
+
+    def __init__(self, qkv, attn_out, ffn1, ffn2):
+        self.weights = (qkv, attn_out, ffn1, ffn2)
+        self.struct = DecoderLayerStruct(*[w.as_struct() for w in self.weights])
+
+    def workspace_halfs(self, tokens):
+        need = 1
+        for w in self.weights:
+            s = w.split_k or splitk_heuristic(w.m, tokens, w.k)
+            need = max(need, s * w.m * tokens)
+        return need
+
+    def forward(self, x, tokens, buffers=None, workspace=None, stream=None):
+        """x: fp16 device tensor, column-major hidden x tokens.  Returns (y, buffers)."""
+        import torch
+
+        qkv, o, f1, f2 = self.weights
+        dev = x.device
+        if buffers is None:
+            buffers = [torch.empty(n * tokens, dtype=torch.float16, device=dev) for n in (qkv.m, o.k, o.m, f1.m, f2.m)]
+        if workspace is None:
+            workspace = torch.empty(self.workspace_halfs(tokens), dtype=torch.float16, device=dev)
+        rc = lib().flashllm_decoder_layer_linears(_stream(stream), ctypes.byref(self.struct), _ptr(x), *[_ptr(b) for b in buffers],
+                                                  tokens, _ptr(workspace))
+        if rc:
+            raise HipError(rc)
+        return buffers[4], buffers

@@ -92,6 +92,52 @@ int flashllm_splitk_heuristic(int M, int N, int K);
  * the contract of reference build/SpMM_API.cuh:33-36. */
 size_t flashllm_workspace_bytes(int M, int N, int Split_K);
 
+/*
+ * One pruned linear layer resident on the GPU: the NZWeights / TileOffsets / SplitK fields the
+ * reference adds to FasterTransformer's DenseWeight (third_party/ft.patch:456-462).
+ * split_k == 0 asks for flashllm_splitk_heuristic at the given token count.
+ */
+typedef struct {
+    const void* nz_weights;   /* device, Compressed_A */
+    const int*  tile_offsets; /* device */
+    int         m;            /* output features (rows of A) */
+    int         k;            /* input features */
+    int         split_k;
+} flashllm_sparse_weight;
+
+/* The four pruned weights of one decoder layer, in the reference's call order
+ * (third_party/ft.patch:1247-1261 QKV, :1328-1340 attention output, :512-525 FFN1, :615-633 FFN2). */
+typedef struct {
+    flashllm_sparse_weight qkv, attn_out, ffn1, ffn2;
+} flashllm_decoder_layer;
+
+/*
+ * Applies the four linears of one decoder layer back to back on `tokens` activations
+ * (column-major, hidden x tokens fp16), all on `stream`, sharing one Reduction_Workspace as the
+ * reference's cublasMMWrapper does (ft.patch:2761-2765, :2822-2847):
+ *     qkv_out  = Wqkv * x                      (3*hidden x tokens)
+ *     attn_out = Wo   * qkv_out[0:hidden, :]   (the attention itself is not part of this library:
+ *                                               the first hidden rows stand in for its output)
+ *     ffn_mid  = relu(W1 * attn_out)
+ *     y        = W2   * ffn_mid
+ * Like the reference's call sites, Split_K falls back to 1 when tokens > 128 (FFN, ft.patch:523)
+ * or tokens > 64 (attention, ft.patch:1454).  attn_in (hidden x tokens) receives the first hidden
+ * rows of every column of qkv_out (a strided copy kernel), because B must be dense column-major.
+ * Buffers: qkv_out qkv.m*tokens, attn_in / attn_out attn_out.k*tokens / attn_out.m*tokens,
+ * ffn_mid ffn1.m*tokens, y ffn2.m*tokens halfs; workspace for the largest Split_K*M*tokens.
+ * Returns a hipError_t as int (hipErrorInvalidValue when the shapes do not chain).
+ */
+int flashllm_decoder_layer_linears(void*                         stream,
+                                   const flashllm_decoder_layer* layer,
+                                   const void*                   x,
+                                   void*                         qkv_out,
+                                   void*                         attn_in,
+                                   void*                         attn_out,
+                                   void*                         ffn_mid,
+                                   void*                         y,
+                                   int                           tokens,
+                                   void*                         Reduction_Workspace);
+
 /* Six-argument file exporter (reference csrc/SpMM_API.cu:500-555) that
  * returns 0 or a FLASHLLM_E_* code instead of exiting. */
 int flashllm_gen_sparse_matrix_bin_file(const char* DenseMatrixFileName,

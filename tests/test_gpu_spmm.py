@@ -247,3 +247,48 @@ def test_nonuniform_rows(product, oracle, torch_gpu):
     for split_k in (1, 6):
         c, _, _ = run_spmm(product, a, b, n, split_k)
         assert_close(c, ref, f"beta rows split_k={split_k}")
+
+
+# --- config 5 flavour: the four linears of a decoder layer, chained --------------------------------
+@pytest.mark.parametrize("tokens", [16, 256])
+def test_decoder_layer_chain(product, oracle, torch_gpu, tokens):
+    """QKV -> (first hidden rows) -> attention output -> FFN1 -> ReLU -> FFN2 on one stream with one
+    workspace; every stage is checked against an fp32 product of the previous stage's fp16 output.
+    tokens = 256 exercises the reference's fallback to Split_K = 1 (ft.patch:523, :1454)."""
+    torch = torch_gpu
+    say(f"decoder layer chain tokens={tokens}")
+    hidden = 512
+    shapes = [(3 * hidden, hidden), (hidden, hidden), (4 * hidden, hidden), (hidden, 4 * hidden)]
+    dense = [synth.sparse_matrix(m, k, 0.8, 20 + i, dist="normal", sigma=0.05) for i, (m, k) in enumerate(shapes)]
+    weights = [product.SparseWeight(a) for a in dense]
+    layer = product.DecoderLayer(*weights)
+    x_h = synth.dense_b(hidden, tokens, 30, dist="normal")
+    x = torch.from_numpy(x_h).cuda()
+    y, bufs = layer.forward(x, tokens)
+    torch.cuda.synchronize()
+    qkv, attn_in, attn_out, ffn_mid, y = [b.cpu().numpy() for b in bufs]
+    qkv = qkv.reshape(tokens, 3 * hidden)
+    ref, _ = oracle.gemm_f32(dense[0], x_h, tokens)
+    assert_close(qkv, ref, "qkv")
+    attn_in = attn_in.reshape(tokens, hidden)
+    assert np.array_equal(attn_in.view(np.uint16), np.ascontiguousarray(qkv[:, :hidden]).view(np.uint16))
+    ref, _ = oracle.gemm_f32(dense[1], attn_in, tokens)
+    attn_out = attn_out.reshape(tokens, hidden)
+    assert_close(attn_out, ref, "attention output")
+    ref, _ = oracle.gemm_f32(dense[2], attn_out, tokens)
+    ffn_mid = ffn_mid.reshape(tokens, 4 * hidden)
+    assert np.all(ffn_mid >= 0)
+    assert_close(ffn_mid, np.maximum(ref, 0), "ffn1 + relu")
+    ref, _ = oracle.gemm_f32(dense[3], ffn_mid, tokens)
+    assert_close(y.reshape(tokens, hidden), ref, "ffn2")
+
+
+def test_decoder_layer_rejects_shapes_that_do_not_chain(product, torch_gpu):
+    torch = torch_gpu
+    a = synth.sparse_matrix(256, 128, 0.8, 1)
+    w = product.SparseWeight(a)
+    layer = product.DecoderLayer(w, w, w, w)  # attention output expects k == hidden == 128 but ffn1.k != attn_out.m
+    x = torch.zeros(128 * 16, dtype=torch.float16, device="cuda")
+    with pytest.raises(product.HipError) as e:
+        layer.forward(x, 16)
+    assert e.value.code == 1

@@ -88,9 +88,9 @@ size_t flashllm_workspace_bytes(int m, int n, int split_k)
 }
 
 // One wave streams one (row tile, K slice, column group) and owns 16 KB of LDS for its tile plus
-// 4 KB per 16 output columns for B staging, so a CU (160 KB) holds 8 / 6 / 4 of them for
-// N <= 16 / 32 / >= 64 (five 32 KB workgroups would need all 160 KB; only four become resident).  The grid should fill those slots on all 256 CUs exactly once, in slices of
-// equal length: a second round of workgroups would run at a fraction of the occupancy.
+// B staging (4 KB at N <= 16 and N = 32, 8 KB at N >= 64), so a CU (160 KB) holds 8 / 8 / 6 of them.
+// The grid should fill those slots on all 256 CUs exactly once, in slices of equal length: a second
+// round of workgroups would run at a fraction of the occupancy.
 int flashllm_splitk_heuristic(int m, int n, int k)
 {
     if (m <= 0 || k <= 0 || n <= 0 || m % 128 || k % 64)
@@ -99,7 +99,7 @@ int flashllm_splitk_heuristic(int m, int n, int k)
     const int  nb         = n <= 16 ? 1 : (n == 32 ? 2 : 4);
     const int  col_groups = n <= 64 ? 1 : n / 64;
     const long units      = static_cast<long>(m / 128) * col_groups;
-    const long slots      = 256L * (nb == 4 ? 4 : 160 / (16 + 4 * nb));
+    const long slots      = 256L * (nb == 4 ? 6 : 8);
     // Largest split that still runs in one round; a second round would run at a fraction of the
     // occupancy (measured at 36864x9216, N=16: 51 us at 7 slices = 2016 waves, 70 us at 8).
     long s_max = slots / units;

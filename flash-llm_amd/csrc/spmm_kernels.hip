@@ -109,7 +109,10 @@ __device__ __forceinline__ void wait_vmcnt()
 // NB: 16-column blocks per wave (1 for N <= 16, 2 for N = 32, 4 for N >= 64).
 // DEPTH: ring slots = 1 KB chunks in flight per wave.
 // BWAIT: a B request followed by at least BWAIT ring loads is awaited with vmcnt(BWAIT).
-template<int NB, int DEPTH, int BWAIT>
+// BBUF: B staging buffers.  Two let the request for tile t+1 go out while tile t's fragments may
+//       still be read; one saves 2*NB KB of LDS per wave (two more resident waves per CU at NB >= 2,
+//       worth 12 % at N = 32 and 27 % at N = 64) and waits for those reads before the request.
+template<int NB, int DEPTH, int BWAIT, int BBUF>
 __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __restrict__ comp,
                                                             const int* __restrict__ offs,
                                                             const _Float16* __restrict__ B,
@@ -120,7 +123,7 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                                                             int split_k)
 {
     __shared__ __attribute__((aligned(16))) uint16_t tile[kTileHalfs];
-    __shared__ __attribute__((aligned(16))) uint32_t bstage[2][2 * NB][256];  // [tile parity][k step, block][lane*4]
+    __shared__ __attribute__((aligned(16))) uint32_t bstage[BBUF][2 * NB][256];  // [tile parity][k step, block][lane*4]
 
     const int lane    = threadIdx.x;
     const int r16     = lane & 15;  // row inside a 16-row block / output column
@@ -168,7 +171,7 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
 #pragma unroll
                 for (int nb = 0; nb < NB; nb++)
                     load_to_lds_16(bptr[nb] + t * kTileCols + ks * 32,
-                                   bstage_lds + (((t & 1) * 2 * NB + ks * NB + nb) << 10));
+                                   bstage_lds + (((t & (BBUF - 1)) * 2 * NB + ks * NB + nb) << 10));
         };
 
         clear_tile(tile, lane);
@@ -203,7 +206,7 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                             else
                                 wait_vmcnt<0>();
                             const char*  base = reinterpret_cast<const char*>(tile);
-                            const uint4* bs   = reinterpret_cast<const uint4*>(&bstage[t & 1][0][0]);
+                            const uint4* bs   = reinterpret_cast<const uint4*>(&bstage[t & (BBUF - 1)][0][0]);
 #pragma unroll
                             for (int ks = 0; ks < 2; ks++) {
                                 half8 bfrag[NB];
@@ -232,6 +235,8 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                         else
                             __builtin_amdgcn_s_setprio(0);
                         if (t < ke) {
+                            if (BBUF == 1)  // the fragments of the tile just multiplied have been read
+                                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                             request_b(t);
                             since   = 0;
                             tile_hi = next_hi;
@@ -354,11 +359,11 @@ __global__ __launch_bounds__(256) void take_rows_kernel(uint4* __restrict__ dst,
     dst[i] = src[static_cast<long>(j) * ld8 + r];
 }
 
-template<int NB, int DEPTH, int BWAIT>
+template<int NB, int DEPTH, int BWAIT, int BBUF>
 int launch_spmm(hipStream_t stream, const void* comp, const int* offs, const void* b, void* out, int m, int n, int k, int split_k, int col_groups)
 {
     const dim3 grid(static_cast<unsigned>(m / kTileRows) * split_k, col_groups, 1);
-    hipLaunchKernelGGL((spmm_stream_kernel<NB, DEPTH, BWAIT>),
+    hipLaunchKernelGGL((spmm_stream_kernel<NB, DEPTH, BWAIT, BBUF>),
                        grid,
                        dim3(kLanes),
                        0,
@@ -381,10 +386,10 @@ extern "C" int flashllm_hip_launch_spmm(
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (n <= 16)
-        return launch_spmm<1, 8, 4>(s, comp, offs, b, out, m, n, k, split_k, 1);
+        return launch_spmm<1, 8, 4, 2>(s, comp, offs, b, out, m, n, k, split_k, 1);
     if (n == 32)
-        return launch_spmm<2, 8, 4>(s, comp, offs, b, out, m, n, k, split_k, 1);
-    return launch_spmm<4, 8, 4>(s, comp, offs, b, out, m, n, k, split_k, n / 64);
+        return launch_spmm<2, 8, 4, 1>(s, comp, offs, b, out, m, n, k, split_k, 1);
+    return launch_spmm<4, 8, 4, 1>(s, comp, offs, b, out, m, n, k, split_k, n / 64);
 }
 
 extern "C" int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws, long mn, int split_k)

@@ -13,12 +13,15 @@
 //   * Each chunk is scattered into the wave's private 128x64 fp16 tile in LDS
 //     at the position stored in the item (the format's XOR-swizzled layout,
 //     reference csrc/SpMM_API.cu:252-261).  When the running vector index
-//     passes TileOffsets[t+1] the tile is complete: the wave reads it back as
-//     16 ds_read_b128 MFMA operands (the swizzle makes every group of eight
-//     lanes hit 32 distinct banks), issues v_mfma_f32_16x16x32_f16 against the
-//     B fragments of that k tile (column-major B already is the MFMA operand
-//     layout: 8 consecutive k per lane), and clears the tile.  Any number of
-//     tiles may end inside one chunk (empty tiles, tiles of a single vector).
+//     passes TileOffsets[t+1] the tile is complete: the wave takes it out of
+//     LDS as 16 MFMA operands of 16 bytes per lane with ds_wrxchg2_rtn_b64,
+//     which returns the operand and leaves zeros behind in one LDS instruction
+//     (the swizzle makes every group of eight lanes hit 32 distinct banks), so
+//     the tile is empty again for the next one without a separate clearing
+//     pass, and issues v_mfma_f32_16x16x32_f16 against the B fragments of that
+//     k tile (column-major B already is the MFMA operand layout: 8 consecutive
+//     k per lane).  Any number of tiles may end inside one chunk (empty tiles,
+//     tiles of a single vector).
 //   * One wave, in-order LDS: no barrier anywhere.
 //
 // Waiting for memory.  The ring loads are the only vector-memory loads the
@@ -29,6 +32,8 @@
 // completes with an explicit vmcnt derived from the number of ring loads
 // issued in between.  The compiler does not know about these loads; extra
 // loads in flight only make its own vmcnt waits stricter, never weaker.
+// The operand exchanges are inline assembly as well (the compiler has no
+// 16-byte LDS exchange), followed by an explicit lgkmcnt(0).
 //
 // splitk_reduce_kernel: the separate reduction over fp16 slabs
 // (reference csrc/Reduction_Kernel.cuh:24-45), 8 bytes per lane per slab, eight slabs in flight.
@@ -100,6 +105,17 @@ __device__ __forceinline__ void load_to_lds_16(const void* g, uint32_t lds_byte_
                  : "memory");
 }
 
+// Returns the 16 bytes at lds_byte_addr and stores zeros there, one LDS instruction.  The result is
+// valid after the next s_waitcnt lgkmcnt(0).
+__device__ __forceinline__ uintx4 take_and_clear_16(uint32_t lds_byte_addr)
+{
+    using uintx2 = uint32_t __attribute__((ext_vector_type(2)));
+    const uintx2 zero = {0u, 0u};
+    uintx4       old;
+    asm volatile("ds_wrxchg2_rtn_b64 %0, %1, %2, %2 offset1:1" : "=v"(old) : "v"(lds_byte_addr), "v"(zero) : "memory");
+    return old;
+}
+
 template<int W>
 __device__ __forceinline__ void wait_vmcnt()
 {
@@ -108,11 +124,12 @@ __device__ __forceinline__ void wait_vmcnt()
 
 // NB: 16-column blocks per wave (1 for N <= 16, 2 for N = 32, 4 for N >= 64).
 // DEPTH: ring slots = 1 KB chunks in flight per wave.
-// BWAIT: a B request followed by at least BWAIT ring loads is awaited with vmcnt(BWAIT).
-// BBUF: B staging buffers.  Two let the request for tile t+1 go out while tile t's fragments may
-//       still be read; one saves 2*NB KB of LDS per wave (two more resident waves per CU at NB >= 2,
-//       worth 12 % at N = 32 and 27 % at N = 64) and waits for those reads before the request.
-template<int NB, int DEPTH, int BWAIT, int BBUF>
+// BWAIT: a B request followed by n ring loads is awaited with vmcnt(min(n, BWAIT)), vmcnt(0) for n < 2.
+//        Short tiles (90 % sparsity and above: three chunks or fewer) would otherwise drain the whole
+//        ring at every tile end.
+// One B staging buffer of 2*NB KB: a second one would let the request for tile t+1 go out before tile
+// t's fragments are read, but costs resident waves (two per CU at NB >= 2) and gains nothing at NB = 1.
+template<int NB, int DEPTH, int BWAIT>
 __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __restrict__ comp,
                                                             const int* __restrict__ offs,
                                                             const _Float16* __restrict__ B,
@@ -123,7 +140,7 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                                                             int split_k)
 {
     __shared__ __attribute__((aligned(16))) uint16_t tile[kTileHalfs];
-    __shared__ __attribute__((aligned(16))) uint32_t bstage[BBUF][2 * NB][256];  // [tile parity][k step, block][lane*4]
+    __shared__ __attribute__((aligned(16))) uint32_t bstage[2 * NB][256];  // [k step, block][lane*4]
 
     const int lane    = threadIdx.x;
     const int r16     = lane & 15;  // row inside a 16-row block / output column
@@ -164,14 +181,15 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
             n        = n < N ? n : N - 1;  // N == 8: lanes 8..15 compute columns nobody stores
             bptr[nb] = B + static_cast<size_t>(n) * K + g * 8;
         }
-        const uint32_t bstage_lds = lds_offset(&bstage[0][0][0]);
+        const uint32_t bstage_lds = lds_offset(&bstage[0][0]);
+        const uint32_t tile_lds   = lds_offset(&tile[0]);
         auto           request_b  = [&](int t) {
 #pragma unroll
             for (int ks = 0; ks < 2; ks++)
 #pragma unroll
                 for (int nb = 0; nb < NB; nb++)
                     load_to_lds_16(bptr[nb] + t * kTileCols + ks * 32,
-                                   bstage_lds + (((t & (BBUF - 1)) * 2 * NB + ks * NB + nb) << 10));
+                                   bstage_lds + ((ks * NB + nb) << 10));
         };
 
         clear_tile(tile, lane);
@@ -201,29 +219,60 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                         scatter_vector(tile, cur);
                     while (tile_hi <= ve) {  // a tile ends inside, or exactly at the end of, this chunk
                         if (tile_hi > tile_lo) {
-                            if (since >= BWAIT)
-                                wait_vmcnt<BWAIT>();
+                            static_assert(BWAIT == 4, "the wait ladder below is written for BWAIT == 4");
+                            if (since >= 4)
+                                wait_vmcnt<4>();
+                            else if (since >= 3)
+                                wait_vmcnt<3>();
+                            else if (since >= 2)
+                                wait_vmcnt<2>();
                             else
                                 wait_vmcnt<0>();
-                            const char*  base = reinterpret_cast<const char*>(tile);
-                            const uint4* bs   = reinterpret_cast<const uint4*>(&bstage[t & (BBUF - 1)][0][0]);
+                            // NB <= 2: all 16 operands in one batch.  NB == 4: one 32-wide k step at a time, which
+                            // keeps the kernel within 256 VGPRs (two waves per SIMD).
+                            constexpr int    kBatch = NB >= 4 ? 1 : 2;
+                            const uint4* bs     = reinterpret_cast<const uint4*>(&bstage[0][0]);
 #pragma unroll
-                            for (int ks = 0; ks < 2; ks++) {
-                                half8 bfrag[NB];
+                            for (int k0 = 0; k0 < 2; k0 += kBatch) {
+                                half8 bfrag[kBatch][NB];
 #pragma unroll
-                                for (int nb = 0; nb < NB; nb++)
-                                    bfrag[nb] = __builtin_bit_cast(half8, bs[(ks * NB + nb) * kLanes + lane]);
-#pragma unroll
-                                for (int rb = 0; rb < 8; rb++) {
-                                    const half8 a = *reinterpret_cast<const half8*>(
-                                        base + rb * (16 * kTileCols * 2) + (ks ? a_off1 : a_off0));
+                                for (int ks = 0; ks < kBatch; ks++)
 #pragma unroll
                                     for (int nb = 0; nb < NB; nb++)
-                                        acc[nb][rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                            a, bfrag[nb], acc[nb][rb], 0, 0, 0);
-                                }
+                                        bfrag[ks][nb] =
+                                            __builtin_bit_cast(half8, bs[((k0 + ks) * NB + nb) * kLanes + lane]);
+                                uintx4 a[kBatch][8];
+#pragma unroll
+                                for (int ks = 0; ks < kBatch; ks++)
+#pragma unroll
+                                    for (int rb = 0; rb < 8; rb++)
+                                        a[ks][rb] = take_and_clear_16(tile_lds + rb * (16 * kTileCols * 2) +
+                                                                      ((k0 + ks) ? a_off1 : a_off0));
+                                // the exchanges above and the B fragment reads have landed
+                                if constexpr (kBatch == 2)
+                                    asm volatile("s_waitcnt lgkmcnt(0)"
+                                                 : "+v"(a[0][0]), "+v"(a[0][1]), "+v"(a[0][2]), "+v"(a[0][3]),
+                                                   "+v"(a[0][4]), "+v"(a[0][5]), "+v"(a[0][6]), "+v"(a[0][7]),
+                                                   "+v"(a[kBatch - 1][0]), "+v"(a[kBatch - 1][1]), "+v"(a[kBatch - 1][2]),
+                                                   "+v"(a[kBatch - 1][3]), "+v"(a[kBatch - 1][4]), "+v"(a[kBatch - 1][5]),
+                                                   "+v"(a[kBatch - 1][6]), "+v"(a[kBatch - 1][7])
+                                                 :
+                                                 : "memory");
+                                else
+                                    asm volatile("s_waitcnt lgkmcnt(0)"
+                                                 : "+v"(a[0][0]), "+v"(a[0][1]), "+v"(a[0][2]), "+v"(a[0][3]),
+                                                   "+v"(a[0][4]), "+v"(a[0][5]), "+v"(a[0][6]), "+v"(a[0][7])
+                                                 :
+                                                 : "memory");
+#pragma unroll
+                                for (int ks = 0; ks < kBatch; ks++)
+#pragma unroll
+                                    for (int rb = 0; rb < 8; rb++)
+#pragma unroll
+                                        for (int nb = 0; nb < NB; nb++)
+                                            acc[nb][rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                                __builtin_bit_cast(half8, a[ks][rb]), bfrag[ks][nb], acc[nb][rb], 0, 0, 0);
                             }
-                            clear_tile(tile, lane);
                         }
                         t++;
                         tile_lo = tile_hi;
@@ -235,9 +284,7 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                         else
                             __builtin_amdgcn_s_setprio(0);
                         if (t < ke) {
-                            if (BBUF == 1)  // the fragments of the tile just multiplied have been read
-                                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                            request_b(t);
+                            request_b(t);  // the fragments of the tile just multiplied were awaited above
                             since   = 0;
                             tile_hi = next_hi;
                             next_hi = toff[t + 2];
@@ -359,11 +406,11 @@ __global__ __launch_bounds__(256) void take_rows_kernel(uint4* __restrict__ dst,
     dst[i] = src[static_cast<long>(j) * ld8 + r];
 }
 
-template<int NB, int DEPTH, int BWAIT, int BBUF>
+template<int NB, int DEPTH, int BWAIT>
 int launch_spmm(hipStream_t stream, const void* comp, const int* offs, const void* b, void* out, int m, int n, int k, int split_k, int col_groups)
 {
     const dim3 grid(static_cast<unsigned>(m / kTileRows) * split_k, col_groups, 1);
-    hipLaunchKernelGGL((spmm_stream_kernel<NB, DEPTH, BWAIT, BBUF>),
+    hipLaunchKernelGGL((spmm_stream_kernel<NB, DEPTH, BWAIT>),
                        grid,
                        dim3(kLanes),
                        0,
@@ -386,10 +433,10 @@ extern "C" int flashllm_hip_launch_spmm(
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (n <= 16)
-        return launch_spmm<1, 8, 4, 2>(s, comp, offs, b, out, m, n, k, split_k, 1);
+        return launch_spmm<1, 8, 4>(s, comp, offs, b, out, m, n, k, split_k, 1);
     if (n == 32)
-        return launch_spmm<2, 8, 4, 1>(s, comp, offs, b, out, m, n, k, split_k, 1);
-    return launch_spmm<4, 8, 4, 1>(s, comp, offs, b, out, m, n, k, split_k, n / 64);
+        return launch_spmm<2, 8, 4>(s, comp, offs, b, out, m, n, k, split_k, 1);
+    return launch_spmm<4, 8, 4>(s, comp, offs, b, out, m, n, k, split_k, n / 64);
 }
 
 extern "C" int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws, long mn, int split_k)

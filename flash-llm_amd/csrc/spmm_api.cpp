@@ -87,19 +87,18 @@ size_t flashllm_workspace_bytes(int m, int n, int split_k)
     return static_cast<size_t>(split_k) * m * n * sizeof(uint16_t);
 }
 
-// One wave streams one (row tile, K slice, column group) and owns 16 KB of LDS for its tile plus
-// B staging (4 KB at N <= 16 and N = 32, 8 KB at N >= 64), so a CU (160 KB) holds 8 / 8 / 6 of them.
-// The grid should fill those slots on all 256 CUs exactly once, in slices of equal length: a second
-// round of workgroups would run at a fraction of the occupancy.
+// One wave streams one (row tile, K slice, column group); its registers allow two waves per SIMD, so a
+// CU holds 8 of them (their 16 KB LDS tiles would allow 10).  The grid should fill those slots on all
+// 256 CUs exactly once, in slices of equal length: a second round of workgroups would run at a
+// fraction of the occupancy.
 int flashllm_splitk_heuristic(int m, int n, int k)
 {
     if (m <= 0 || k <= 0 || n <= 0 || m % 128 || k % 64)
         return 1;
     const int  kt         = k / 64;
-    const int  nb         = n <= 16 ? 1 : (n == 32 ? 2 : 4);
     const int  col_groups = n <= 64 ? 1 : n / 64;
     const long units      = static_cast<long>(m / 128) * col_groups;
-    const long slots      = 256L * (nb == 4 ? 6 : 8);
+    const long slots      = 256L * 8;
     // Largest split that still runs in one round; a second round would run at a fraction of the
     // occupancy (measured at 36864x9216, N=16: 51 us at 7 slices = 2016 waves, 70 us at 8).
     long s_max = slots / units;

@@ -24,16 +24,16 @@
 //     tiles of a single vector).
 //   * One wave, in-order LDS: no barrier anywhere.
 //
-// Waiting for memory.  The ring loads are the only vector-memory loads the
-// compiler sees, and every path through a ring stage issues exactly one, so
-// its wait before a slot is used is the exact vmcnt(DEPTH-1).  The B fragments
-// of the next tile travel global -> LDS with global_load_lds_dwordx4 issued
-// from inline assembly when the tile is opened, and are awaited when it
-// completes with an explicit vmcnt derived from the number of ring loads
-// issued in between.  The compiler does not know about these loads; extra
-// loads in flight only make its own vmcnt waits stricter, never weaker.
-// The operand exchanges are inline assembly as well (the compiler has no
-// 16-byte LDS exchange), followed by an explicit lgkmcnt(0).
+// Waiting for memory.  Every path through a ring stage issues exactly one
+// ring load, so the compiler's wait before a slot is used is the exact
+// vmcnt(DEPTH-1).  The B fragments of a k tile (column-major B already is the
+// MFMA operand layout, 16 bytes per lane per fragment) are loaded straight
+// into registers when the tile is opened and first used when it completes;
+// the compiler places those waits as well.  Staging B through LDS instead
+// (global_load_lds_dwordx4) measured the same at N <= 32 and slower at
+// N = 64, where its 8 KB per wave cost two resident waves per CU.
+// The operand exchanges are inline assembly (the compiler has no 16-byte LDS
+// exchange), followed by an explicit lgkmcnt(0).
 //
 // splitk_reduce_kernel: the separate reduction over fp16 slabs
 // (reference csrc/Reduction_Kernel.cuh:24-45), 8 bytes per lane per slab, eight slabs in flight.
@@ -90,21 +90,6 @@ __device__ __forceinline__ uint32_t lds_offset(const void* p)
     return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) void*)(p)));
 }
 
-// 16 bytes per lane, global -> LDS at lds_byte_addr + lane*16, without passing through registers.
-// Counted by vmcnt like any load, but invisible to the compiler's wait insertion.
-__device__ __forceinline__ void load_to_lds_16(const void* g, uint32_t lds_byte_addr)
-{
-    uint32_t saved;
-    asm volatile("s_mov_b32 %0, m0\n\t"
-                 "s_mov_b32 m0, %2\n\t"
-                 "s_nop 0\n\t"
-                 "global_load_lds_dwordx4 %1, off\n\t"
-                 "s_mov_b32 m0, %0\n\t"
-                 : "=&s"(saved)
-                 : "v"(g), "s"(lds_byte_addr)
-                 : "memory");
-}
-
 // Returns the 16 bytes at lds_byte_addr and stores zeros there, one LDS instruction.  The result is
 // valid after the next s_waitcnt lgkmcnt(0).
 __device__ __forceinline__ uintx4 take_and_clear_16(uint32_t lds_byte_addr)
@@ -116,20 +101,10 @@ __device__ __forceinline__ uintx4 take_and_clear_16(uint32_t lds_byte_addr)
     return old;
 }
 
-template<int W>
-__device__ __forceinline__ void wait_vmcnt()
-{
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(W) : "memory");
-}
-
 // NB: 16-column blocks per wave (1 for N <= 16, 2 for N = 32, 4 for N >= 64).
-// DEPTH: ring slots = 1 KB chunks in flight per wave.
-// BWAIT: a B request followed by n ring loads is awaited with vmcnt(min(n, BWAIT)), vmcnt(0) for n < 2.
-//        Short tiles (90 % sparsity and above: three chunks or fewer) would otherwise drain the whole
-//        ring at every tile end.
-// One B staging buffer of 2*NB KB: a second one would let the request for tile t+1 go out before tile
-// t's fragments are read, but costs resident waves (two per CU at NB >= 2) and gains nothing at NB = 1.
-template<int NB, int DEPTH, int BWAIT>
+// DEPTH: ring slots = 1 KB chunks in flight per wave (8; 6 at NB = 4, which keeps that instance within
+// 256 VGPRs = two waves per SIMD).
+template<int NB, int DEPTH>
 __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __restrict__ comp,
                                                             const int* __restrict__ offs,
                                                             const _Float16* __restrict__ B,
@@ -140,7 +115,6 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                                                             int split_k)
 {
     __shared__ __attribute__((aligned(16))) uint16_t tile[kTileHalfs];
-    __shared__ __attribute__((aligned(16))) uint32_t bstage[2 * NB][256];  // [k step, block][lane*4]
 
     const int lane    = threadIdx.x;
     const int r16     = lane & 15;  // row inside a 16-row block / output column
@@ -181,15 +155,14 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
             n        = n < N ? n : N - 1;  // N == 8: lanes 8..15 compute columns nobody stores
             bptr[nb] = B + static_cast<size_t>(n) * K + g * 8;
         }
-        const uint32_t bstage_lds = lds_offset(&bstage[0][0]);
-        const uint32_t tile_lds   = lds_offset(&tile[0]);
-        auto           request_b  = [&](int t) {
+        const uint32_t tile_lds = lds_offset(&tile[0]);
+        half8          bfrag[2][NB];  // B fragments of the open tile
+        auto           load_b = [&](int t) {
 #pragma unroll
             for (int ks = 0; ks < 2; ks++)
 #pragma unroll
                 for (int nb = 0; nb < NB; nb++)
-                    load_to_lds_16(bptr[nb] + t * kTileCols + ks * 32,
-                                   bstage_lds + ((ks * NB + nb) << 10));
+                    bfrag[ks][nb] = *reinterpret_cast<const half8*>(bptr[nb] + t * kTileCols + ks * 32);
         };
 
         clear_tile(tile, lane);
@@ -203,8 +176,7 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
             ring[d] = uint4{0u, 0u, 0u, 0u};
 
         int t = kb, tile_lo = vbeg, tile_hi = toff[kb + 1], next_hi = toff[kb + 2];
-        int since = 0;  // ring loads issued after the latest B request
-        request_b(t);
+        load_b(t);
 
         // Chunks -DEPTH .. -1 only fill the ring: none of their lanes reaches tile_lo, and a tile can
         // only "end" there when it is empty.
@@ -219,28 +191,11 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                         scatter_vector(tile, cur);
                     while (tile_hi <= ve) {  // a tile ends inside, or exactly at the end of, this chunk
                         if (tile_hi > tile_lo) {
-                            static_assert(BWAIT == 4, "the wait ladder below is written for BWAIT == 4");
-                            if (since >= 4)
-                                wait_vmcnt<4>();
-                            else if (since >= 3)
-                                wait_vmcnt<3>();
-                            else if (since >= 2)
-                                wait_vmcnt<2>();
-                            else
-                                wait_vmcnt<0>();
                             // NB <= 2: all 16 operands in one batch.  NB == 4: one 32-wide k step at a time, which
                             // keeps the kernel within 256 VGPRs (two waves per SIMD).
                             constexpr int    kBatch = NB >= 4 ? 1 : 2;
-                            const uint4* bs     = reinterpret_cast<const uint4*>(&bstage[0][0]);
 #pragma unroll
                             for (int k0 = 0; k0 < 2; k0 += kBatch) {
-                                half8 bfrag[kBatch][NB];
-#pragma unroll
-                                for (int ks = 0; ks < kBatch; ks++)
-#pragma unroll
-                                    for (int nb = 0; nb < NB; nb++)
-                                        bfrag[ks][nb] =
-                                            __builtin_bit_cast(half8, bs[((k0 + ks) * NB + nb) * kLanes + lane]);
                                 uintx4 a[kBatch][8];
 #pragma unroll
                                 for (int ks = 0; ks < kBatch; ks++)
@@ -248,7 +203,7 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                                     for (int rb = 0; rb < 8; rb++)
                                         a[ks][rb] = take_and_clear_16(tile_lds + rb * (16 * kTileCols * 2) +
                                                                       ((k0 + ks) ? a_off1 : a_off0));
-                                // the exchanges above and the B fragment reads have landed
+                                // the exchanges above have landed
                                 if constexpr (kBatch == 2)
                                     asm volatile("s_waitcnt lgkmcnt(0)"
                                                  : "+v"(a[0][0]), "+v"(a[0][1]), "+v"(a[0][2]), "+v"(a[0][3]),
@@ -271,21 +226,26 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
 #pragma unroll
                                         for (int nb = 0; nb < NB; nb++)
                                             acc[nb][rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                                __builtin_bit_cast(half8, a[ks][rb]), bfrag[ks][nb], acc[nb][rb], 0, 0, 0);
+                                                __builtin_bit_cast(half8, a[ks][rb]), bfrag[k0 + ks][nb], acc[nb][rb], 0, 0, 0);
                             }
                         }
                         t++;
                         tile_lo = tile_hi;
                         // The SIMD's arbiter serves its older wave first, which leaves the younger of the two
                         // resident waves about 17 % slower; taking turns at raised priority, one tile each,
-                        // evens their finishing times.
-                        if ((t ^ wave_slot) & 1)
-                            __builtin_amdgcn_s_setprio(1);
+                        // evens their finishing times.  The tile counters of the two waves are not in step:
+                        // the younger wave's raised level is the higher one, so it wins when both are raised
+                        // as the older one wins when neither is.
+                        if ((t ^ wave_slot) & 1) {
+                            if (wave_slot)
+                                __builtin_amdgcn_s_setprio(2);
+                            else
+                                __builtin_amdgcn_s_setprio(1);
+                        }
                         else
                             __builtin_amdgcn_s_setprio(0);
                         if (t < ke) {
-                            request_b(t);  // the fragments of the tile just multiplied were awaited above
-                            since   = 0;
+                            load_b(t);
                             tile_hi = next_hi;
                             next_hi = toff[t + 2];
                             if (v >= tile_lo && v < tile_hi)  // the rest of this chunk opens the next tile
@@ -301,7 +261,6 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                     int vn  = v + DEPTH * kLanes;
                     vn      = vn < vlast ? vn : vlast;
                     ring[d] = load_stream(comp + vn);
-                    since++;
                 }
             }
         }
@@ -406,11 +365,11 @@ __global__ __launch_bounds__(256) void take_rows_kernel(uint4* __restrict__ dst,
     dst[i] = src[static_cast<long>(j) * ld8 + r];
 }
 
-template<int NB, int DEPTH, int BWAIT>
+template<int NB, int DEPTH>
 int launch_spmm(hipStream_t stream, const void* comp, const int* offs, const void* b, void* out, int m, int n, int k, int split_k, int col_groups)
 {
     const dim3 grid(static_cast<unsigned>(m / kTileRows) * split_k, col_groups, 1);
-    hipLaunchKernelGGL((spmm_stream_kernel<NB, DEPTH, BWAIT>),
+    hipLaunchKernelGGL((spmm_stream_kernel<NB, DEPTH>),
                        grid,
                        dim3(kLanes),
                        0,
@@ -433,10 +392,10 @@ extern "C" int flashllm_hip_launch_spmm(
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (n <= 16)
-        return launch_spmm<1, 8, 4>(s, comp, offs, b, out, m, n, k, split_k, 1);
+        return launch_spmm<1, 8>(s, comp, offs, b, out, m, n, k, split_k, 1);
     if (n == 32)
-        return launch_spmm<2, 8, 4>(s, comp, offs, b, out, m, n, k, split_k, 1);
-    return launch_spmm<4, 8, 4>(s, comp, offs, b, out, m, n, k, split_k, n / 64);
+        return launch_spmm<2, 8>(s, comp, offs, b, out, m, n, k, split_k, 1);
+    return launch_spmm<4, 6>(s, comp, offs, b, out, m, n, k, split_k, n / 64);
 }
 
 extern "C" int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws, long mn, int split_k)

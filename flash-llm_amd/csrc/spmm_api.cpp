@@ -80,6 +80,36 @@ int flashllm_spmm_splitk(void*       stream,
     return flashllm_hip_launch_reduce(stream, c, ws, static_cast<long>(m) * n, split_k);
 }
 
+int flashllm_device_tile_offsets(void* stream, const void* a, int m, int k, int* offs, long long* nnz_padded)
+{
+    if (!a || !offs || (reinterpret_cast<uintptr_t>(a) & 15u))
+        return FLASHLLM_E_ARG;
+    if (m <= 0 || k <= 0 || m % 128 || k % 64)
+        return FLASHLLM_E_SHAPE;
+    int rc = flashllm_hip_launch_tile_offsets(stream, a, m, k, offs);
+    if (rc || !nnz_padded)
+        return rc;
+    const size_t tiles   = static_cast<size_t>(m / 128) * (k / 64);
+    int          vectors = 0;
+    hipStream_t  s       = static_cast<hipStream_t>(stream);
+    hipError_t   e       = hipMemcpyAsync(&vectors, offs + tiles, sizeof(int), hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess)
+        e = hipStreamSynchronize(s);
+    if (e != hipSuccess)
+        return static_cast<int>(e);
+    *nnz_padded = 4LL * vectors;
+    return 0;
+}
+
+int flashllm_device_compress(void* stream, const void* a, int m, int k, const int* offs, void* comp)
+{
+    if (!a || !offs || !comp || (reinterpret_cast<uintptr_t>(a) & 15u) || (reinterpret_cast<uintptr_t>(comp) & 15u))
+        return FLASHLLM_E_ARG;
+    if (m <= 0 || k <= 0 || m % 128 || k % 64)
+        return FLASHLLM_E_SHAPE;
+    return flashllm_hip_launch_encode(stream, a, m, k, offs, comp);
+}
+
 size_t flashllm_workspace_bytes(int m, int n, int split_k)
 {
     if (split_k <= 1 || m <= 0 || n <= 0)

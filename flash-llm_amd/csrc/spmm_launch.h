@@ -29,6 +29,13 @@ int flashllm_hip_launch_relu(void* stream, void* x, long n);
 // dst[j*rows + i] = src[j*src_ld + i] for i < rows, j < cols (rows % 8 == 0, src_ld % 8 == 0).
 int flashllm_hip_launch_take_rows(void* stream, void* dst, const void* src, int rows, int cols, int src_ld);
 
+// offs[0..tiles+1] = TileOffsets of the device-resident dense matrix a (M x K halfs, 16-byte aligned,
+// M % 128 == 0, K % 64 == 0): a count kernel and an in-place prefix sum.
+int flashllm_hip_launch_tile_offsets(void* stream, const void* a, int m, int k, int* offs);
+
+// out[offs[t]*4 ...] = the packed nonzeros of tile t in the reference's reordered layout.
+int flashllm_hip_launch_encode(void* stream, const void* a, int m, int k, const int* offs, void* out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -44,6 +44,8 @@ SIGNATURES = {
     "flashllm_spmm_splitk": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int]),
     "flashllm_spmm_partials": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int]),
     "flashllm_splitk_reduce": (ctypes.c_int, [_vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "flashllm_device_tile_offsets": (ctypes.c_int, [_vp, _vp, ctypes.c_int, ctypes.c_int, _vp, ctypes.POINTER(ctypes.c_longlong)]),
+    "flashllm_device_compress": (ctypes.c_int, [_vp, _vp, ctypes.c_int, ctypes.c_int, _vp, _vp]),
     "flashllm_splitk_heuristic": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "flashllm_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "flashllm_decoder_layer_linears": (ctypes.c_int, [_vp, ctypes.POINTER(DecoderLayerStruct), _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp]),
@@ -164,6 +166,29 @@ def splitk_reduce(c, workspace, m, n, split_k, stream=None):
     rc = lib().flashllm_splitk_reduce(_stream(stream), _ptr(c), _ptr(workspace), m, n, split_k)
     if rc:
         raise HipError(rc)
+
+
+def device_compress(a_dev, stream=None):
+    """Tiled-CSL compression of a device-resident fp16 matrix (torch tensor M x K) on the GPU.
+    Returns (Compressed_A int32 tensor[NNZ_padded], TileOffsets int32 tensor[tiles+2]), both on the
+    device, with the bytes InitSparseMatrixA_API produces on the host."""
+    import torch
+
+    if a_dev.dim() != 2 or a_dev.dtype != torch.float16 or not a_dev.is_contiguous():
+        raise TypeError("A must be a contiguous 2-D float16 device tensor")
+    m, k = a_dev.shape
+    if m <= 0 or k <= 0 or m % 128 or k % 64:
+        raise CompressError(-1)
+    offs = torch.empty((m // 128) * (k // 64) + 2, dtype=torch.int32, device=a_dev.device)
+    nnz = ctypes.c_longlong(0)
+    rc = lib().flashllm_device_tile_offsets(_stream(stream), _ptr(a_dev), m, k, _ptr(offs), ctypes.byref(nnz))
+    if rc:
+        raise CompressError(rc) if rc < 0 else HipError(rc)
+    comp = torch.empty(max(int(nnz.value), 4), dtype=torch.int32, device=a_dev.device)
+    rc = lib().flashllm_device_compress(_stream(stream), _ptr(a_dev), m, k, _ptr(offs), _ptr(comp))
+    if rc:
+        raise CompressError(rc) if rc < 0 else HipError(rc)
+    return comp[: int(nnz.value)], offs
 
 
 class SparseWeight:

@@ -7,6 +7,7 @@ this build is measured on.  Prints one JSON line per case.
     python flash-llm_amd/sweep.py hidden12k  # hidden-12288 projections, Beta(2,8) row densities, N = 32
     python flash-llm_amd/sweep.py square     # 9216 x 9216, N = 16, Split_K {1,2,4,8,heuristic}
     python flash-llm_amd/sweep.py layers     # four chained linears per layer, hidden 9216, 16 tokens, 8 layers
+    python flash-llm_amd/sweep.py compress   # Tiled-CSL compression of 36864 x 9216: host threads vs the device-side compressor
 
 Every case reports ms per call, dense-equivalent TFLOPS (2MNK/t, kernel_benchmark/spmm_test.cu:314-316),
 algorithmic GB/s and its fraction of the 8 TB/s HBM peak, a dense fp16 GEMM of the same shape through
@@ -134,6 +135,37 @@ def main():
                           "ms_all_layers": ms, "ms_per_layer": per_layer, "tflops": flops / ms / 1e9,
                           "weight_GB_compressed": comp_bytes / 1e9, "weight_GB_dense": dense_bytes / 1e9,
                           "alg_GBps": comp_bytes / ms / 1e6, "frac_hbm": comp_bytes / ms / 1e6 / HBM_PEAK}), flush=True)
+    elif what == "compress":
+        # Tiled-CSL compression of the headline weight: host (threaded, and on one thread as the reference
+        # runs it) against the device-side compressor on a device-resident matrix.
+
+        m, k = 36864, 9216
+        a = synth.sparse_matrix(m, k, 0.8, 0, dist="normal", sigma=0.02, threads=threads)
+        t0 = time.perf_counter()
+        items, offsets = F.init_sparse_matrix_a(a, threads=threads)
+        t_host = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        F.init_sparse_matrix_a(a, threads=1)
+        t_host1 = time.perf_counter() - t0
+        F.lib().flashllm_set_compress_threads(0)
+        a_dev = torch.from_numpy(a).cuda()
+        comp, offs = F.device_compress(a_dev)
+        torch.cuda.synchronize()
+        same = bool(np.array_equal(comp.cpu().numpy().view(np.uint32), items) and np.array_equal(offs.cpu().numpy(), offsets))
+
+        def both(i):
+            F.lib().flashllm_device_tile_offsets(None, a_dev.data_ptr(), m, k, offs.data_ptr(), None)
+            F.lib().flashllm_device_compress(None, a_dev.data_ptr(), m, k, offs.data_ptr(), comp.data_ptr())
+
+        ms = timed(torch, both, steps=20, settle_ms=100)
+        ms_offsets = timed(torch, lambda i: F.lib().flashllm_device_tile_offsets(None, a_dev.data_ptr(), m, k, offs.data_ptr(), None),
+                           steps=20, settle_ms=100)
+        moved = 2 * 2.0 * m * k + 4.0 * items.size + 2 * 4.0 * offsets.size
+        print(json.dumps({"case": "Tiled-CSL compression 36864x9216 80%", "host_threads": threads, "host_s": t_host,
+                          "host_1thread_s": t_host1, "device_ms": ms, "device_offsets_ms": ms_offsets,
+                          "device_encode_ms": ms - ms_offsets, "device_bytes_moved_MB": moved / 1e6,
+                          "device_GBps": moved / ms / 1e6, "frac_hbm": moved / ms / 1e6 / HBM_PEAK,
+                          "bit_identical_to_host": same}), flush=True)
     else:
         sys.exit(__doc__)
 

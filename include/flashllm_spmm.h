@@ -88,6 +88,28 @@ int flashllm_splitk_reduce(void* stream, void* C, const void* Reduction_Workspac
  */
 int flashllm_splitk_heuristic(int M, int N, int K);
 
+/*
+ * Tiled-CSL compression on the GPU for a dense matrix that is already in
+ * device memory: the bytes of flashllm_init_sparse_matrix_a (reference
+ * InitSparseMatrixA_API, csrc/SpMM_API.cu:163-360, which runs on the host on
+ * one thread), produced by one wave per 128x64 tile.  Two calls, because the
+ * caller owns the output allocation:
+ *
+ *  flashllm_device_tile_offsets fills TileOffsets (device, (M/128)*(K/64)+2
+ *  ints) and, when NNZ_padded is not NULL, waits for the stream and stores the
+ *  number of packed items (TileOffsets[last]*4) there, so that the caller can
+ *  allocate Compressed_A (4 bytes per item, 16-byte aligned);
+ *
+ *  flashllm_device_compress writes Compressed_A (device) from A and the
+ *  TileOffsets of the first call, asynchronously on the stream.
+ *
+ * A: device pointer, row-major M x K halfs, 16-byte aligned; M % 128 == 0,
+ * K % 64 == 0.  Returns 0, a negative FLASHLLM_E_* code or a positive
+ * hipError_t value.
+ */
+int flashllm_device_tile_offsets(void* stream, const void* A, int M, int K, int* TileOffsets, long long* NNZ_padded);
+int flashllm_device_compress(void* stream, const void* A, int M, int K, const int* TileOffsets, void* Compressed_A);
+
 /* Bytes the caller must provide as Reduction_Workspace (0 when Split_K == 1);
  * the contract of reference build/SpMM_API.cuh:33-36. */
 size_t flashllm_workspace_bytes(int M, int N, int Split_K);

@@ -117,9 +117,10 @@ size_t flashllm_workspace_bytes(int m, int n, int split_k)
     return static_cast<size_t>(split_k) * m * n * sizeof(uint16_t);
 }
 
-// One wave streams one (row tile, K slice, column group); its registers allow two waves per SIMD, so a
-// CU holds 8 of them (their 16 KB LDS tiles would allow 10).  The grid should fill those slots on all
-// 256 CUs exactly once, in slices of equal length: a second round of workgroups would run at a
+// One wave streams one (row tile, K slice, column group).  Two waves per SIMD, 8 per CU, is what the
+// kernel is tuned for and what its registers allow at N >= 32; at N <= 16 a CU could hold 10 (16 KB LDS
+// tiles), but a ninth wave per CU already measures 5 % slower.  The grid should fill those slots on
+// all 256 CUs exactly once, in slices of equal length: a second round of workgroups would run at a
 // fraction of the occupancy.
 int flashllm_splitk_heuristic(int m, int n, int k)
 {
@@ -130,7 +131,7 @@ int flashllm_splitk_heuristic(int m, int n, int k)
     const long units      = static_cast<long>(m / 128) * col_groups;
     const long slots      = 256L * 8;
     // Largest split that still runs in one round; a second round would run at a fraction of the
-    // occupancy (measured at 36864x9216, N=16: 51 us at 7 slices = 2016 waves, 70 us at 8).
+    // occupancy (measured at 36864x9216, N=16: 46 us at 7 slices = 2016 waves, 49 us at 8, 62 us at 9).
     long s_max = slots / units;
     if (s_max > 32)
         s_max = 32;  // workspace sizes in existing callers assume at most 32 slabs

@@ -15,10 +15,11 @@
 //   * The drain's tail-then-main fill and its last-in-first-out write-out
 //     (csrc/SpMM_API.cu:306-346) map j to one output index.
 //
-// One wave64 per 128x64 tile: the tile is laid out bank-major in LDS, bank
-// fills and first-zero positions come from 64-lane ballots, and each nonzero
-// writes itself to its final place.  Three kernels: vectors per tile, an
-// in-place prefix sum (TileOffsets), the encoder.
+// One workgroup of four waves per 128x64 tile: the tile is laid out bank-major
+// in LDS, each wave takes eight banks, bank fills and first-zero positions
+// come from 64-lane ballots, and each nonzero writes itself to its final
+// place.  Three kernels: vectors per tile, an in-place prefix sum
+// (TileOffsets), the encoder.
 #include "spmm_launch.h"
 
 #include <hip/hip_runtime.h>
@@ -72,62 +73,70 @@ __global__ __launch_bounds__(kLanes) void count_tiles_kernel(const uint16_t* __r
         offs[t + 1] = (n + 3) / 4;
 }
 
-// in place: offs[0] = 0, offs[t + 1] = sum of the counts up to tile t, offs[tiles + 1] = offs[tiles]
+// in place: offs[0] = 0, offs[t + 1] = sum of the counts up to tile t, offs[tiles + 1] = offs[tiles].
+// One workgroup; every thread sums a contiguous run of tiles, the 1024 run totals are scanned once.
 __global__ __launch_bounds__(1024) void scan_offsets_kernel(int* __restrict__ offs, int tiles)
 {
     __shared__ int part[1024];
-    __shared__ int carry;
     const int      tid = threadIdx.x;
-    if (tid == 0)
-        carry = 0;
+    const int      run = (tiles + 1023) / 1024;
+    const int      lo  = tid * run < tiles ? tid * run : tiles;
+    const int      hi  = lo + run < tiles ? lo + run : tiles;
+    int            sum = 0;
+    for (int i = lo; i < hi; i++)
+        sum += offs[i + 1];
+    part[tid] = sum;
     __syncthreads();
-    for (int base = 0; base < tiles; base += 1024) {
-        const int i = base + tid;
-        part[tid]   = i < tiles ? offs[i + 1] : 0;
+    for (int s = 1; s < 1024; s <<= 1) {
+        const int add = tid >= s ? part[tid - s] : 0;
         __syncthreads();
-        for (int s = 1; s < 1024; s <<= 1) {
-            const int add = tid >= s ? part[tid - s] : 0;
-            __syncthreads();
-            part[tid] += add;
-            __syncthreads();
-        }
-        const int c = carry;
-        if (i < tiles)
-            offs[i + 1] = c + part[tid];
-        __syncthreads();
-        if (tid == 0)
-            carry = c + part[1023];
+        part[tid] += add;
         __syncthreads();
     }
-    if (tid == 0) {
+    int acc = part[tid] - sum;  // total of the runs before this one
+    for (int i = lo; i < hi; i++) {
+        acc += offs[i + 1];
+        offs[i + 1] = acc;
+    }
+    if (tid == 1023) {
         offs[0]         = 0;
-        offs[tiles + 1] = carry;
+        offs[tiles + 1] = part[1023];
     }
 }
 
-__global__ __launch_bounds__(kLanes) void encode_tiles_kernel(const uint16_t* __restrict__ a,
-                                                             int k,
-                                                             int tiles_per_row,
-                                                             const int* __restrict__ offs,
-                                                             uint32_t* __restrict__ out)
+// One workgroup of four waves per tile; wave w owns banks 8w .. 8w+7.
+constexpr int kEncodeWaves  = 4;
+constexpr int kBanksPerWave = kBanks / kEncodeWaves;
+
+__global__ __launch_bounds__(kLanes* kEncodeWaves) void encode_tiles_kernel(const uint16_t* __restrict__ a,
+                                                                            int k,
+                                                                            int tiles_per_row,
+                                                                            const int* __restrict__ offs,
+                                                                            uint32_t* __restrict__ out)
 {
     __shared__ __attribute__((aligned(16))) uint16_t vals[kBanks][kPerBank];  // bank-major: [bank][2*row + (column & 1)]
     __shared__ int                                   fill_s[kBanks];
+    __shared__ int                                   first_zero_s[kBanks];    // in-tile position of the bank's first zero, -1: none
+    __shared__ int                                   pad_s[3][3];             // bank, height, position of each padding item
+    __shared__ int                                   npad_s;
     __shared__ int                                   above[kMaxFill + 2];     // items higher than h, over all banks
     __shared__ uint32_t                              reach[kMaxFill + 2];     // banks holding at least h items
+    __shared__ uint16_t                              tail_dest[4 * kBanks];   // output index of the first 4*rem pops
 
     const int       t    = blockIdx.x;
-    const int       lane = threadIdx.x;
+    const int       tid  = threadIdx.x;
+    const int       lane = tid & (kLanes - 1);
+    const int       wave = tid >> 6;
     const uint16_t* base = tile_base(a, k, tiles_per_row, t);
 
     // Element (m, n) lives at swizzled column sw = n ^ ((m % 8) << 3) (csrc/SpMM_API.cu:252-256): the
     // 8-column chunk c of row m becomes chunk c ^ (m % 8), order inside the chunk unchanged, so the four
-    // 32-bit words of a lane's 16 bytes are the four banks (c ^ (m % 8)) * 4 + w at in-bank index 2m, 2m+1.
-#pragma unroll 4
-    for (int it = 0; it < kTileRows / 8; it++) {
-        const int   m  = it * 8 + (lane >> 3);
-        const uint4 v  = *reinterpret_cast<const uint4*>(base + static_cast<size_t>(m) * k + (lane & 7) * 8);
-        const int   b0 = ((lane & 7) ^ (m & 7)) * 4;
+    // 32-bit words of a thread's 16 bytes are the four banks (c ^ (m % 8)) * 4 + w at in-bank index 2m, 2m+1.
+#pragma unroll
+    for (int it = 0; it < kTileRows / 32; it++) {
+        const int   m  = it * 32 + (tid >> 3);
+        const uint4 v  = *reinterpret_cast<const uint4*>(base + static_cast<size_t>(m) * k + (tid & 7) * 8);
+        const int   b0 = ((tid & 7) ^ (m & 7)) * 4;
         *reinterpret_cast<uint32_t*>(&vals[b0 + 0][2 * m]) = v.x;
         *reinterpret_cast<uint32_t*>(&vals[b0 + 1][2 * m]) = v.y;
         *reinterpret_cast<uint32_t*>(&vals[b0 + 2][2 * m]) = v.z;
@@ -135,10 +144,10 @@ __global__ __launch_bounds__(kLanes) void encode_tiles_kernel(const uint16_t* __
     }
     __syncthreads();
 
-    // fill and first zero (in scan order) of every bank; lane b keeps bank b's
-    int fill = 0, first_zero = -1, nnz = 0;
-    for (int b = 0; b < kBanks; b++) {
-        int cnt = 0, fz = -1;
+    // fill and first zero (in scan order) of this wave's banks
+    for (int bi = 0; bi < kBanksPerWave; bi++) {
+        const int b   = wave * kBanksPerWave + bi;
+        int       cnt = 0, fz = -1;
 #pragma unroll
         for (int q = 0; q < kPerBank / kLanes; q++) {
             const uint64_t mask = __builtin_amdgcn_ballot_w64(keeps(vals[b][q * kLanes + lane]));
@@ -146,37 +155,56 @@ __global__ __launch_bounds__(kLanes) void encode_tiles_kernel(const uint16_t* __
             if (fz < 0 && ~mask != 0)
                 fz = q * kLanes + __builtin_ctzll(~mask);
         }
-        nnz += cnt;
-        if (lane == b) {
-            fill       = cnt;
-            first_zero = fz < 0 ? -1 : (fz >> 1) * kTileCols + 2 * b + (fz & 1);  // in-tile position of that zero
+        if (lane == 0) {
+            fill_s[b]       = cnt;
+            first_zero_s[b] = fz < 0 ? -1 : (fz >> 1) * kTileCols + 2 * b + (fz & 1);
         }
     }
-
-    // Padding to a multiple of four: each padding item goes on top of the emptiest bank (lowest index
-    // on ties) at that bank's first zero position, value 0 (csrc/SpMM_API.cu:274-287).
-    const int pad = (4 - nnz % 4) % 4;
-    int       pad_bank[3] = {0, 0, 0}, pad_height[3] = {1, 1, 1}, pad_pos[3] = {0, 0, 0};
-    for (int p = 0; p < pad; p++) {
-        int key = lane < kBanks ? (fill << 5) | lane : 0x7fffffff;
-#pragma unroll
-        for (int s = 32; s >= 1; s >>= 1) {
-            const int other = __shfl_xor(key, s);
-            key             = other < key ? other : key;
-        }
-        const int b  = key & 31;
-        const int fz = __shfl(first_zero, b);
-        pad_bank[p]   = b;
-        pad_height[p] = (key >> 5) + 1;
-        pad_pos[p]    = fz < 0 ? 0 : fz;  // the emptiest bank holds fewer than 256 items, so it has a zero
-        if (lane == b)
-            fill++;
-    }
-    if (lane < kBanks)
-        fill_s[lane] = fill;
     __syncthreads();
 
-    for (int h = lane; h < kMaxFill + 2; h += kLanes) {
+    // Padding to a multiple of four: each padding item goes on top of the emptiest bank (lowest index
+    // on ties) at that bank's first zero position, value 0 (csrc/SpMM_API.cu:274-287).  Wave 0 decides.
+    if (wave == 0) {
+        int fill = lane < kBanks ? fill_s[lane] : 0;
+        int nnz  = fill;
+#pragma unroll
+        for (int s = 32; s >= 1; s >>= 1)
+            nnz += __shfl_xor(nnz, s);
+        const int pad = (4 - nnz % 4) % 4;
+        for (int p = 0; p < pad; p++) {
+            int key = lane < kBanks ? (fill << 5) | lane : 0x7fffffff;
+#pragma unroll
+            for (int s = 32; s >= 1; s >>= 1) {
+                const int other = __shfl_xor(key, s);
+                key             = other < key ? other : key;
+            }
+            const int b = key & 31;
+            if (lane == b) {
+                const int fz = first_zero_s[b];
+                pad_s[p][0]  = b;
+                pad_s[p][1]  = fill + 1;
+                pad_s[p][2]  = fz < 0 ? 0 : fz;  // the emptiest bank holds fewer than 256 items, so it has a zero
+                fill++;
+            }
+        }
+        if (lane < kBanks)
+            fill_s[lane] = fill;
+        if (lane == 0)
+            npad_s = pad;
+    }
+    __syncthreads();
+
+    int count = 0, top = 0;
+    for (int b = 0; b < kBanks; b++) {
+        const int f = fill_s[b];
+        count += f;
+        top = f > top ? f : top;
+    }
+    const int vectors    = count / 4;
+    const int rep        = vectors / kBanks, rem = vectors % kBanks;
+    const int tail_items = rem * 4;
+
+    for (int h = tid; h <= top + 1; h += kLanes * kEncodeWaves) {
         int      g = 0;
         uint32_t r = 0;
         for (int b = 0; b < kBanks; b++) {
@@ -187,21 +215,17 @@ __global__ __launch_bounds__(kLanes) void encode_tiles_kernel(const uint16_t* __
         above[h] = g;
         reach[h] = r;
     }
+    // the first 4*rem pops are drained first, lane-major per pass; each lane is written back to front
+    if (tid < tail_items)
+        tail_dest[tid] = static_cast<uint16_t>(rep * 4 * kBanks + (tid % rem) * 4 + (3 - tid / rem));
     __syncthreads();
 
-    const int count      = nnz + pad;
-    const int vectors    = count / 4;
-    const int rep        = vectors / kBanks, rem = vectors % kBanks;
-    const int tail_items = rem * 4;
-    uint32_t* out_tile   = out + static_cast<size_t>(offs[t]) * 4;
-
-    auto emit = [&](int b, int h, uint32_t item) {
+    uint32_t* out_tile = out + static_cast<size_t>(offs[t]) * 4;
+    auto      emit     = [&](int b, int h, uint32_t item) {
         const int j = above[h] + __builtin_popcount(reach[h] & ((1u << b) - 1u));
         int       d;
         if (j < tail_items) {
-            // drained first, lane-major per pass; each lane is written back to front
-            const int pass = j / rem, ln = j % rem;
-            d              = rep * 4 * kBanks + ln * 4 + (3 - pass);
+            d = tail_dest[j];
         }
         else {
             const int q    = j - tail_items;
@@ -213,8 +237,9 @@ __global__ __launch_bounds__(kLanes) void encode_tiles_kernel(const uint16_t* __
             out_tile[d] = item;
     };
 
-    for (int b = 0; b < kBanks; b++) {
-        int below = 0;
+    for (int bi = 0; bi < kBanksPerWave; bi++) {
+        const int b     = wave * kBanksPerWave + bi;
+        int       below = 0;
 #pragma unroll
         for (int q = 0; q < kPerBank / kLanes; q++) {
             const int      i    = q * kLanes + lane;
@@ -229,12 +254,8 @@ __global__ __launch_bounds__(kLanes) void encode_tiles_kernel(const uint16_t* __
             below += __builtin_popcountll(mask);
         }
     }
-    if (lane < pad) {
-        const int p = lane;
-        emit(p == 0 ? pad_bank[0] : (p == 1 ? pad_bank[1] : pad_bank[2]),
-             p == 0 ? pad_height[0] : (p == 1 ? pad_height[1] : pad_height[2]),
-             static_cast<uint32_t>(p == 0 ? pad_pos[0] : (p == 1 ? pad_pos[1] : pad_pos[2])) << 16);
-    }
+    if (tid < npad_s)
+        emit(pad_s[tid][0], pad_s[tid][1], static_cast<uint32_t>(pad_s[tid][2]) << 16);
 }
 
 }  // namespace
@@ -258,7 +279,7 @@ extern "C" int flashllm_hip_launch_encode(void* stream, const void* a, int m, in
     const int tiles         = (m / kTileRows) * tiles_per_row;
     hipLaunchKernelGGL(encode_tiles_kernel,
                        dim3(tiles),
-                       dim3(kLanes),
+                       dim3(kLanes * kEncodeWaves),
                        0,
                        static_cast<hipStream_t>(stream),
                        static_cast<const uint16_t*>(a),

@@ -13,6 +13,10 @@ PKG = os.path.join(ROOT, "flash-llm_amd")
 
 @pytest.fixture(scope="module")
 def dropin(product, tmp_path_factory):
+    src = os.path.join(ROOT, "tests", "cxx", "dropin.cpp")
+    prebuilt = os.path.join(ROOT, "tests", "cxx", "dropin.bin")  # what __graft_entry__.build() leaves
+    if os.path.exists(prebuilt) and os.path.getmtime(prebuilt) >= os.path.getmtime(src):
+        return prebuilt
     exe = str(tmp_path_factory.mktemp("cxx") / "dropin")
     cmd = ["/opt/rocm/bin/hipcc", "-O2", "--offload-arch=gfx950", "-I", os.path.join(ROOT, "include"),
            os.path.join(ROOT, "tests", "cxx", "dropin.cpp"), "-o", exe, "-L", PKG, "-lSpMM_API", f"-Wl,-rpath,{PKG}",

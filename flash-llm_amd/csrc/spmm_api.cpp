@@ -59,7 +59,7 @@ int flashllm_splitk_reduce(void* stream, void* c, const void* ws, int m, int n, 
 {
     if (!c || !ws || m <= 0 || n <= 0 || split_k < 1 || (static_cast<long>(m) * n) % 4)
         return hipErrorInvalidValue;
-    return flashllm_hip_launch_reduce(stream, c, ws, static_cast<long>(m) * n, split_k);
+    return flashllm_hip_launch_reduce(stream, c, ws, static_cast<long>(m) * n, split_k, 0);
 }
 
 int flashllm_spmm_splitk(void*       stream,
@@ -77,7 +77,7 @@ int flashllm_spmm_splitk(void*       stream,
     int rc = flashllm_spmm_partials(stream, comp, offs, b, c, m, n, k, ws, split_k);
     if (rc || split_k == 1)
         return rc;
-    return flashllm_hip_launch_reduce(stream, c, ws, static_cast<long>(m) * n, split_k);
+    return flashllm_hip_launch_reduce(stream, c, ws, static_cast<long>(m) * n, split_k, 0);
 }
 
 int flashllm_device_tile_offsets(void* stream, const void* a, int m, int k, int* offs, long long* nnz_padded)
@@ -194,10 +194,13 @@ int flashllm_decoder_layer_linears(void*                         stream,
     rc = linear(o, attn_in, attn_out, 64);
     if (rc)
         return rc;
-    rc = linear(f1, attn_out, ffn_mid, 128);
+    // FFN1 with the ReLU folded into its reduction when there is one
+    const int s1 = split(f1, 128);
+    rc = flashllm_spmm_partials(stream, f1.nz_weights, f1.tile_offsets, attn_out, ffn_mid, f1.m, tokens, f1.k, ws, s1);
     if (rc)
         return rc;
-    rc = flashllm_hip_launch_relu(stream, ffn_mid, static_cast<long>(f1.m) * tokens);
+    rc = s1 > 1 ? flashllm_hip_launch_reduce(stream, ffn_mid, ws, static_cast<long>(f1.m) * tokens, s1, 1)
+                : flashllm_hip_launch_relu(stream, ffn_mid, static_cast<long>(f1.m) * tokens);
     if (rc)
         return rc;
     return linear(f2, ffn_mid, y, 128);

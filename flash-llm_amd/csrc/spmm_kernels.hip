@@ -296,6 +296,8 @@ __device__ __forceinline__ void add_slab(float (&s)[4], const uint2 v)
 // C[e] = rn16(sum over slabs, in slab order, of float(ws[s*MN + e])).  Eight bytes per lane and up to
 // eight slabs in flight per lane: the slabs are small (M*N halfs), so the kernel is latency bound and
 // wants many independent loads rather than wide ones.
+// RELU: the sums go through max(x, 0) before rounding (the activation after FFN1, saving a pass over C)
+template<bool RELU>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(uint2* __restrict__ c,
                                                            const uint2* __restrict__ ws,
                                                            long n4,
@@ -340,7 +342,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(uint2* __restrict__ 
     half4 h;
 #pragma unroll
     for (int j = 0; j < 4; j++)
-        h[j] = static_cast<_Float16>(s[j]);
+        h[j] = static_cast<_Float16>(RELU && !(s[j] > 0.f) ? 0.f : s[j]);
     c[i] = __builtin_bit_cast(uint2, h);
 }
 
@@ -398,18 +400,17 @@ extern "C" int flashllm_hip_launch_spmm(
     return launch_spmm<4, 6>(s, comp, offs, b, out, m, n, k, split_k, n / 64);
 }
 
-extern "C" int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws, long mn, int split_k)
+extern "C" int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws, long mn, int split_k, int relu)
 {
-    const long n4 = mn / 4;
-    hipLaunchKernelGGL(splitk_reduce_kernel,
-                       dim3(static_cast<unsigned>((n4 + 255) / 256)),
-                       dim3(256),
-                       0,
-                       static_cast<hipStream_t>(stream),
-                       static_cast<uint2*>(c),
-                       static_cast<const uint2*>(ws),
-                       n4,
-                       split_k);
+    const long     n4 = mn / 4;
+    const dim3     grid(static_cast<unsigned>((n4 + 255) / 256));
+    hipStream_t    s  = static_cast<hipStream_t>(stream);
+    uint2*         cp = static_cast<uint2*>(c);
+    const uint2*   wp = static_cast<const uint2*>(ws);
+    if (relu)
+        hipLaunchKernelGGL(splitk_reduce_kernel<true>, grid, dim3(256), 0, s, cp, wp, n4, split_k);
+    else
+        hipLaunchKernelGGL(splitk_reduce_kernel<false>, grid, dim3(256), 0, s, cp, wp, n4, split_k);
     return static_cast<int>(hipGetLastError());
 }
 

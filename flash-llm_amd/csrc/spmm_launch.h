@@ -20,8 +20,8 @@ int flashllm_hip_launch_spmm(void*       stream,
                              int         k,
                              int         split_k);
 
-// c[e] = rn16(sum_s float(ws[s*mn + e])); requires mn % 4 == 0.
-int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws, long mn, int split_k);
+// c[e] = rn16(sum_s float(ws[s*mn + e])), through max(., 0) first when relu != 0; requires mn % 4 == 0.
+int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws, long mn, int split_k, int relu);
 
 // x[i] = max(x[i], 0) over n halfs (n % 8 == 0): the activation between FFN1 and FFN2.
 int flashllm_hip_launch_relu(void* stream, void* x, long n);

@@ -1,0 +1,201 @@
+// Kernel benchmark with the command line and report layout of the reference's
+// kernel_benchmark/spmm_test.cu (main at :45-834, report at :799-823, PrintPerformance in
+// spmm_test_utils.h:157-164):
+//
+//     ./spmm_test M K N Sparsity SplitK        (SplitK 0 = the library's heuristic)
+//
+// Times, with events around back-to-back launches after warm-up (spmm_test_utils.h:21-22), the dense
+// fp16 GEMM of the same shape through rocBLAS (the reference's cuBLAS tensor-core line), SpMM_SplitK_API
+// on the reordered Tiled-CSL weights ("FlashLLM_v2") and on the not reordered ones ("FlashLLM_v1"),
+// and prints ms, 2*M*N*K/t TFLOPs and the summed absolute difference to the dense result.
+// The other baselines of the reference (cuSPARSE, Sputnik, SparTA) are separate libraries, not part of this one.
+// Iteration counts: environment FLASHLLM_WARMUP (default 100) and FLASHLLM_ITERS (default 2000).
+#include "SpMM_API.h"
+#include "flashllm_spmm.h"
+
+#include <hip/hip_runtime.h>
+#include <rocblas/rocblas.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#define CHECK_HIP(x)                                                                              \
+    do {                                                                                          \
+        hipError_t e_ = (x);                                                                      \
+        if (e_ != hipSuccess) {                                                                   \
+            printf("Error in spmm_test.cpp: line %d: %s\n", __LINE__, hipGetErrorString(e_));     \
+            exit(1);                                                                              \
+        }                                                                                         \
+    } while (0)
+
+namespace {
+
+uint64_t splitmix(uint64_t x)
+{
+    x += 0x9e3779b97f4a7c15ull;
+    x = (x ^ (x >> 30)) * 0xbf58476d1ce4e5b9ull;
+    x = (x ^ (x >> 27)) * 0x94d049bb133111ebull;
+    return x ^ (x >> 31);
+}
+
+uint16_t to_half_bits(float f)
+{
+    const _Float16 h = static_cast<_Float16>(f);
+    uint16_t       u;
+    memcpy(&u, &h, 2);
+    return u;
+}
+
+float from_half_bits(uint16_t u)
+{
+    _Float16 h;
+    memcpy(&h, &u, 2);
+    return static_cast<float>(h);
+}
+
+int env_int(const char* name, int fallback)
+{
+    const char* v = getenv(name);
+    return v && atoi(v) > 0 ? atoi(v) : fallback;
+}
+
+void print_line(const char* kernel, float ms, double flops, double error)
+{
+    printf("%-10s \t -> \t\t Time/ms: %5.3f \t Performance/TFLOPs: %4.2f \t TotalError: %.2lf\n",
+           kernel, ms, flops / (ms * 1e-3) / 1e12, error);
+}
+
+double total_error(const std::vector<uint16_t>& a, const std::vector<uint16_t>& b)
+{
+    double e = 0;
+    for (size_t i = 0; i < a.size(); i++)
+        e += fabs(static_cast<double>(from_half_bits(a[i])) - from_half_bits(b[i]));
+    return e;
+}
+
+template<typename F>
+float time_ms(hipStream_t stream, int warmup, int iters, F&& launch)
+{
+    hipEvent_t e0, e1;
+    CHECK_HIP(hipEventCreate(&e0));
+    CHECK_HIP(hipEventCreate(&e1));
+    for (int i = 0; i < warmup; i++)
+        launch();
+    CHECK_HIP(hipEventRecord(e0, stream));
+    for (int i = 0; i < iters; i++)
+        launch();
+    CHECK_HIP(hipEventRecord(e1, stream));
+    CHECK_HIP(hipEventSynchronize(e1));
+    float ms = 0;
+    CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
+    CHECK_HIP(hipEventDestroy(e0));
+    CHECK_HIP(hipEventDestroy(e1));
+    return ms / iters;
+}
+
+}  // namespace
+
+int main(int argc, char** argv)
+{
+    if (argc != 6) {
+        printf("Wrong Inputs! Correct input format: ./spmm_test M K N Sparsity SplitK\n");
+        return 1;
+    }
+    const int M = atoi(argv[1]), K = atoi(argv[2]), N = atoi(argv[3]), sparsity = atoi(argv[4]);
+    int       split_k = atoi(argv[5]);
+    if (M <= 0 || K <= 0 || N <= 0 || M % 128 || K % 64 || sparsity < 0 || sparsity > 100) {
+        printf("Wrong Inputs! M must be a multiple of 128, K of 64, Sparsity a percentage\n");
+        return 1;
+    }
+    if (split_k <= 0)
+        split_k = flashllm_splitk_heuristic(M, N, K);
+    const int    warmup = env_int("FLASHLLM_WARMUP", 100), iters = env_int("FLASHLLM_ITERS", 2000);
+    const double flops  = 2.0 * M * N * K;
+
+    // A: row-major M x K, pruned at random; B: column-major K x N
+    std::vector<uint16_t> a_h(static_cast<size_t>(M) * K), b_h(static_cast<size_t>(K) * N);
+    for (size_t i = 0; i < a_h.size(); i++) {
+        const uint64_t r = splitmix(i);
+        a_h[i] = (r % 100) < static_cast<uint64_t>(sparsity) ? 0 : to_half_bits(((r >> 20) % 2001) / 1000.0f - 1.0f);
+    }
+    for (size_t i = 0; i < b_h.size(); i++)
+        b_h[i] = to_half_bits((splitmix(i + (1ull << 40)) % 2001) / 1000.0f - 1.0f);
+
+    hipStream_t stream = nullptr;  // the reference times on the default stream
+    const size_t c_halfs = static_cast<size_t>(M) * N;
+    half *       a_d, *b_d, *c_d, *ws_d;
+    CHECK_HIP(hipMalloc(&a_d, a_h.size() * 2));
+    CHECK_HIP(hipMalloc(&b_d, b_h.size() * 2));
+    CHECK_HIP(hipMalloc(&c_d, c_halfs * 2));
+    CHECK_HIP(hipMalloc(&ws_d, c_halfs * 2 * split_k));
+    CHECK_HIP(hipMemcpy(a_d, a_h.data(), a_h.size() * 2, hipMemcpyHostToDevice));
+    CHECK_HIP(hipMemcpy(b_d, b_h.data(), b_h.size() * 2, hipMemcpyHostToDevice));
+
+    // ---- dense: C (column-major M x N) = A * B, A given row-major = op(A) = T with lda = K ----------
+    printf("Launching rocBLAS...\n");
+    rocblas_handle handle;
+    if (rocblas_create_handle(&handle) != rocblas_status_success) {
+        printf("Error in spmm_test.cpp: rocblas_create_handle failed\n");
+        return 1;
+    }
+    rocblas_set_stream(handle, stream);
+    const float alpha = 1.0f, beta = 0.0f;
+    auto        dense = [&]() {
+        rocblas_gemm_ex(handle, rocblas_operation_transpose, rocblas_operation_none, M, N, K, &alpha, a_d,
+                        rocblas_datatype_f16_r, K, b_d, rocblas_datatype_f16_r, K, &beta, c_d, rocblas_datatype_f16_r, M,
+                        c_d, rocblas_datatype_f16_r, M, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+    };
+    const float ms_dense = time_ms(stream, warmup, iters, dense);
+    std::vector<uint16_t> c_dense(c_halfs), c_sparse(c_halfs);
+    CHECK_HIP(hipMemcpy(c_dense.data(), c_d, c_halfs * 2, hipMemcpyDeviceToHost));
+    rocblas_destroy_handle(handle);
+    CHECK_HIP(hipFree(a_d));
+
+    // ---- Flash-LLM: reordered (v2) and not reordered (v1) Tiled-CSL ----------------------------------
+    float  ms_sparse[2]  = {0, 0};
+    double err_sparse[2] = {0, 0};
+    for (int variant = 0; variant < 2; variant++) {
+        printf(variant == 0 ? "Launching Flash-LLM...\n"
+                            : "Launching Flash-LLM without Ahead of Time Sparse Data Reordering...\n");
+        uint32_t* comp_h = nullptr;
+        int*      offs_h = nullptr;
+        half*     a_half = reinterpret_cast<half*>(a_h.data());
+        const int num_offsets = variant == 0 ? InitSparseMatrixA_API(a_half, M, N, K, &comp_h, &offs_h)
+                                             : InitSparseMatrixA_API_NoReorder(a_half, M, N, K, &comp_h, &offs_h);
+        if (num_offsets < 0)
+            return 1;
+        const size_t nnz = static_cast<size_t>(offs_h[num_offsets - 1]) * 4;
+        uint32_t*    comp_d;
+        int*         offs_d;
+        CHECK_HIP(hipMalloc(&comp_d, (nnz ? nnz : 4) * sizeof(uint32_t)));
+        CHECK_HIP(hipMalloc(&offs_d, num_offsets * sizeof(int)));
+        CHECK_HIP(hipMemcpy(comp_d, comp_h, nnz * sizeof(uint32_t), hipMemcpyHostToDevice));
+        CHECK_HIP(hipMemcpy(offs_d, offs_h, num_offsets * sizeof(int), hipMemcpyHostToDevice));
+        free(comp_h);
+        free(offs_h);
+        CHECK_HIP(hipMemset(c_d, 0, c_halfs * 2));
+        auto sparse = [&]() {
+            (void)SpMM_SplitK_API(stream, nullptr, reinterpret_cast<const uint4*>(comp_d), offs_d, b_d, c_d, M, N, K, ws_d, split_k);
+        };
+        ms_sparse[variant] = time_ms(stream, warmup, iters, sparse);
+        CHECK_HIP(hipGetLastError());
+        CHECK_HIP(hipMemcpy(c_sparse.data(), c_d, c_halfs * 2, hipMemcpyDeviceToHost));
+        err_sparse[variant] = total_error(c_dense, c_sparse);
+        CHECK_HIP(hipFree(comp_d));
+        CHECK_HIP(hipFree(offs_d));
+    }
+
+    printf("******************************************Problem Size******************************************\n");
+    printf("M: %d N: %d K: %d Pruning Rate: %d SplitK: %d\n", M, N, K, sparsity, split_k);
+    print_line("rocBLAS_TC", ms_dense, flops, 0.0);
+    print_line("FlashLLM_v1", ms_sparse[1], flops, err_sparse[1]);
+    print_line("FlashLLM_v2", ms_sparse[0], flops, err_sparse[0]);
+    CHECK_HIP(hipFree(b_d));
+    CHECK_HIP(hipFree(c_d));
+    CHECK_HIP(hipFree(ws_d));
+    return 0;
+}

@@ -7,6 +7,7 @@
 //   <name>.OutputSizes.bin  int32 NNZ(padded), int32 NumOffsets
 #include "flashllm_spmm.h"
 
+#include <climits>
 #include <cstdio>
 #include <cstdlib>
 #include <vector>
@@ -53,10 +54,17 @@ extern "C" int flashllm_gen_sparse_matrix_bin_file(const char* dense_name,
     const int n_off   = flashllm_init_sparse_matrix_a(dense.data(), M, K, &nz, &offsets);
     if (n_off < 0)
         return n_off;
-    const int nnz     = offsets[n_off - 1] * 4;
-    const int sizes[2] = {nnz, n_off};
-    const bool ok = write_all(sizes_name, sizes, sizeof(sizes)) && write_all(nz_name, nz, sizeof(uint32_t) * nnz)
-                    && write_all(offsets_name, offsets, sizeof(int) * n_off);
+    // .OutputSizes.bin holds NNZ as an int32 (reference csrc/SpMM_API.cu:533,551): a weight whose padded
+    // item count does not fit cannot be described by the format
+    const long long nnz = 4LL * offsets[n_off - 1];
+    if (nnz > INT_MAX) {
+        flashllm_free(nz);
+        flashllm_free(offsets);
+        return FLASHLLM_E_SHAPE;
+    }
+    const int  sizes[2] = {static_cast<int>(nnz), n_off};
+    const bool ok = write_all(sizes_name, sizes, sizeof(sizes)) && write_all(nz_name, nz, sizeof(uint32_t) * static_cast<size_t>(nnz))
+                    && write_all(offsets_name, offsets, sizeof(int) * static_cast<size_t>(n_off));
     flashllm_free(nz);
     flashllm_free(offsets);
     return ok ? 0 : FLASHLLM_E_IO;

@@ -14,6 +14,7 @@
 #include "flashllm_spmm.h"
 
 #include <atomic>
+#include <climits>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -174,8 +175,14 @@ void for_each_tile(size_t tiles, F&& body)
                 body(t);
         }
     };
-    for (int w = 1; w < workers; w++)
-        pool.emplace_back(run);
+    // a thread that cannot be created is simply left out: the others (at least this one) drain the tiles
+    try {
+        pool.reserve(workers);
+        for (int w = 1; w < workers; w++)
+            pool.emplace_back(run);
+    }
+    catch (...) {
+    }
     run();
     for (auto& th : pool)
         th.join();
@@ -201,9 +208,13 @@ int compress(const uint16_t* A, int M, int K, uint32_t** comp_out, int** offs_ou
         const uint16_t* tile = A + (t / tc) * kTileRows * ld + (t % tc) * kTileCols;
         offs[t + 1]          = count_tile(tile, ld);
     });
-    std::vector<uint8_t> pad(tiles);
-    long long            running = 0;  // in items
-    offs[0]                      = 0;
+    uint8_t* pad = static_cast<uint8_t*>(std::malloc(tiles));
+    if (!pad) {
+        std::free(offs);
+        return FLASHLLM_E_NOMEM;
+    }
+    long long running = 0;  // in items
+    offs[0]           = 0;
     for (size_t t = 0; t < tiles; t++) {
         const int nnz = offs[t + 1];
         pad[t]        = static_cast<uint8_t>((kVec - nnz % kVec) % kVec);
@@ -211,8 +222,14 @@ int compress(const uint16_t* A, int M, int K, uint32_t** comp_out, int** offs_ou
         offs[t + 1] = static_cast<int>(running / kVec);
     }
     offs[tiles + 1] = static_cast<int>(running / kVec);  // the trailing empty tile
+    if (running / kVec > INT_MAX) {  // TileOffsets are int32 counts of 16-byte vectors (reference csrc/SpMM_API.cu:226,349)
+        std::free(pad);
+        std::free(offs);
+        return FLASHLLM_E_SHAPE;
+    }
     uint32_t* comp  = static_cast<uint32_t*>(std::malloc(sizeof(uint32_t) * static_cast<size_t>(running > 0 ? running : 1)));
     if (!comp) {
+        std::free(pad);
         std::free(offs);
         return FLASHLLM_E_NOMEM;
     }
@@ -229,6 +246,7 @@ int compress(const uint16_t* A, int M, int K, uint32_t** comp_out, int** offs_ou
             encode_tile_scan(tile, ld, pad[t], dst);
         }
     });
+    std::free(pad);
     if (!ok) {
         std::free(comp);
         std::free(offs);
@@ -243,15 +261,27 @@ int compress(const uint16_t* A, int M, int K, uint32_t** comp_out, int** offs_ou
 
 extern "C" {
 
+// No exception may cross the C boundary: what little can still throw in there (the thread pool's
+// bookkeeping) is reported as an allocation failure.
 int flashllm_init_sparse_matrix_a(const uint16_t* A_h, int M, int K, uint32_t** Compressed_A, int** TileOffsets)
 {
-    return compress(A_h, M, K, Compressed_A, TileOffsets, true);
+    try {
+        return compress(A_h, M, K, Compressed_A, TileOffsets, true);
+    }
+    catch (...) {
+        return FLASHLLM_E_NOMEM;
+    }
 }
 
 int flashllm_init_sparse_matrix_a_noreorder(
     const uint16_t* A_h, int M, int K, uint32_t** Compressed_A, int** TileOffsets)
 {
-    return compress(A_h, M, K, Compressed_A, TileOffsets, false);
+    try {
+        return compress(A_h, M, K, Compressed_A, TileOffsets, false);
+    }
+    catch (...) {
+        return FLASHLLM_E_NOMEM;
+    }
 }
 
 void flashllm_free(void* p)

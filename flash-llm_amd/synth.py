@@ -27,24 +27,33 @@ def _key(seed, stream):
     return _mix(_mix(np.uint64(seed)) ^ np.uint64(stream))
 
 
-def uniform01(seed, stream, start, count):
-    """float64 in [0,1) for element indices start .. start+count-1."""
-    idx = np.arange(start, start + count, dtype=np.uint64)
+def uniform01_at(seed, stream, idx):
+    """float64 in [0,1) for the element indices in idx (uint64 array)."""
     with np.errstate(over="ignore"):
         z = _mix(idx * _GOLDEN + _key(seed, stream))
     return (z >> np.uint64(11)).astype(np.float64) * (1.0 / 9007199254740992.0)
 
 
-def _values(seed, stream, start, count, dist, sigma):
+def uniform01(seed, stream, start, count):
+    """float64 in [0,1) for element indices start .. start+count-1."""
+    return uniform01_at(seed, stream, np.arange(start, start + count, dtype=np.uint64))
+
+
+def _values_at(seed, stream, idx, dist, sigma):
+    """The value of every element index in idx: a function of (seed, stream, index) alone."""
     if dist == "uniform":  # U[-1, 1]
-        return uniform01(seed, stream, start, count) * 2.0 - 1.0
+        return uniform01_at(seed, stream, idx) * 2.0 - 1.0
     if dist == "normal":  # Box-Muller
-        u1 = uniform01(seed, stream, start, count)
-        u2 = uniform01(seed, stream + 1, start, count)
+        u1 = uniform01_at(seed, stream, idx)
+        u2 = uniform01_at(seed, stream + 1, idx)
         return sigma * np.sqrt(-2.0 * np.log1p(-u1)) * np.cos(2.0 * np.pi * u2)
     if dist == "ones":  # the reference's own test data
-        return np.ones(count)
+        return np.ones(idx.size)
     raise ValueError(dist)
+
+
+def _values(seed, stream, start, count, dist, sigma):
+    return _values_at(seed, stream, np.arange(start, start + count, dtype=np.uint64), dist, sigma)
 
 
 def row_keep_ratio(m, seed, mean=0.2):
@@ -64,14 +73,17 @@ def sparse_matrix(m, k, sparsity, seed, dist="uniform", sigma=0.02, row_beta=Fal
     def block(r0):
         r1 = min(m, r0 + step)
         n = (r1 - r0) * k
-        vals = _values(seed, 1, r0 * k, n, dist, sigma)
         u = uniform01(seed, 3, r0 * k, n)
         if keep_row is None:
             keep = u < (1.0 - sparsity)
         else:
             keep = u.reshape(r1 - r0, k) < keep_row[r0:r1, None]
             keep = keep.reshape(-1)
-        out[r0:r1] = np.where(keep, vals, 0.0).astype(np.float16).reshape(r1 - r0, k)
+        # values only where the mask keeps them: an element's value depends on its index alone
+        kept = np.flatnonzero(keep)
+        blk = np.zeros(n, dtype=np.float16)
+        blk[kept] = _values_at(seed, 1, kept.astype(np.uint64) + np.uint64(r0 * k), dist, sigma).astype(np.float16)
+        out[r0:r1] = blk.reshape(r1 - r0, k)
 
     starts = list(range(0, m, step))
     if threads > 1 and len(starts) > 1:

@@ -8,13 +8,19 @@ resident in HBM.  Steps rotate over several device copies of Compressed_A (272 M
 256 MB Infinity Cache together) so every launch streams its weights from HBM.
 
 Prints one JSON line; `value` = dense-equivalent TFLOPS = 2*M*N*K / t (the reference's formula,
-kernel_benchmark/spmm_test.cu:314-316).  `roofline` is for the SpMM kernel alone, timed live with
-events on the launch stream; `cpu_baseline` times the CPU oracle (compression on one thread, fp32 GEMM
-on all host cores) on the same workload and is a reported figure, not a target.
+kernel_benchmark/spmm_test.cu:314-316) of the whole call.  `roofline`: `frac` (= `kernel_frac`) is for the
+dominant kernel alone (the SpMM kernel, timed live with events on the launch stream in a second loop
+without the reduction); `whole_call_frac` is the same algorithmic bytes over the time of the whole call,
+the figure `value` corresponds to.  `traffic` is the HBM bytes per SpMM-kernel launch measured with
+rocprofv3 counters, read from the summary under profiles/ whose workload line matches this run (null when
+none does).  `cpu_baseline` times the CPU oracle (compression on one thread, fp32 GEMM on all host cores)
+on the same workload and is a reported figure, not a target.
 """
 import argparse
+import glob
 import json
 import os
+import re
 import sys
 import time
 
@@ -23,11 +29,19 @@ sys.path.insert(0, os.path.join(ROOT, "flash-llm_amd"))
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per SpMM-kernel launch at the default Split_K, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs of this command, each scaled by what the same counter reads for the 256 MiB copy of
-# --calibrate-copy (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); profiles/ holds the summary.  Shapes that
-# were not profiled report null.
-MEASURED_TRAFFIC_BYTES = {(36864, 9216, 16, 7): 284841436}
+
+def measured_traffic(m, k, n, split_k, nnz_padded):
+    """HBM bytes per SpMM-kernel launch from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary of this
+    very workload under profiles/ (each counter scaled by what it reads for a plain 256 MiB copy): the
+    summary carries a line `traffic_bytes_per_launch: <bytes> M=.. K=.. N=.. split_k=.. nnz_padded=..`.
+    Returns (bytes, file) or (None, None) when no summary matches this run."""
+    pat = re.compile(r"traffic_bytes_per_launch:\s*(\d+)\s+M=(\d+)\s+K=(\d+)\s+N=(\d+)\s+split_k=(\d+)\s+nnz_padded=(\d+)")
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.md"))):
+        with open(path) as f:
+            for hit in pat.finditer(f.read()):
+                if tuple(int(x) for x in hit.groups()[1:]) == (m, k, n, split_k, nnz_padded):
+                    return int(hit.group(1)), os.path.relpath(path, ROOT)
+    return None, None
 
 
 def algorithmic_bytes(nnz_padded, m, n, k):
@@ -155,6 +169,8 @@ def main():
     alg = algorithmic_bytes(nnz, m, n, k)
     flops = 2.0 * m * n * k
     achieved = alg / (ms_kernel * 1e-3) / 1e9
+    traffic, traffic_source = measured_traffic(m, k, n, split_k, nnz)
+    xcd = F.xcd_of_workgroups((m // 128) * split_k)
     out = {
         "metric": "dense-equiv TFLOPS + % HBM roofline, M=36864 K=9216 N=16, 80% sparse fp16",
         "value": flops / (ms_step * 1e-3) / 1e12,
@@ -162,6 +178,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_ms": args.settle_ms,
         "ms_per_step": ms_step,
         "higher_is_better": True,
         "scaling": "weak",
@@ -179,9 +196,12 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((m, k, n, split_k)) if abs(args.sparsity - 0.8) < 1e-9 else None,
+            "traffic": traffic,
+            "traffic_source": traffic_source,
             "kernel": "spmm_stream_kernel",
             "kernel_ms": ms_kernel,
+            "kernel_frac": achieved / HBM_PEAK_GBS,
+            "whole_call_frac": alg / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "algorithmic_bytes": alg,
         },
         "whole_call": {
@@ -190,6 +210,8 @@ def main():
             "reduction_ms": max(ms_step - ms_kernel, 0.0),
         },
         "max_rel_err_sampled_rows": rel_err,
+        # the placement of slices and reduction workgroups counts on workgroup w running on XCD w % 8
+        "xcd_round_robin": bool((xcd == xcd[[i % 8 for i in range(xcd.size)]]).all()),
     }
 
     if args.calibrate_copy:

@@ -34,6 +34,15 @@ int check_shape(const void* comp, const int* offs, const void* b, const void* c,
     return hipSuccess;
 }
 
+// The reduction behind a SpMM launch of this shape: by blocks of C on the XCD that holds their slabs when the
+// layout allows it (always, for shapes the SpMM kernel takes, unless C is only 8-byte aligned).
+int reduce_slabs(void* stream, void* c, const void* ws, int m, int n, int split_k, int relu)
+{
+    if (m % 128 == 0 && supported_n(n) && reinterpret_cast<uintptr_t>(c) % 16 == 0 && reinterpret_cast<uintptr_t>(ws) % 16 == 0)
+        return flashllm_hip_launch_reduce_blocks(stream, c, ws, m, n, split_k, relu);
+    return flashllm_hip_launch_reduce(stream, c, ws, static_cast<long>(m) * n, split_k, relu);
+}
+
 }  // namespace
 
 extern "C" {
@@ -59,7 +68,7 @@ int flashllm_splitk_reduce(void* stream, void* c, const void* ws, int m, int n, 
 {
     if (!c || !ws || m <= 0 || n <= 0 || split_k < 1 || (static_cast<long>(m) * n) % 4)
         return hipErrorInvalidValue;
-    return flashllm_hip_launch_reduce(stream, c, ws, static_cast<long>(m) * n, split_k, 0);
+    return reduce_slabs(stream, c, ws, m, n, split_k, 0);
 }
 
 int flashllm_spmm_splitk(void*       stream,
@@ -77,7 +86,7 @@ int flashllm_spmm_splitk(void*       stream,
     int rc = flashllm_spmm_partials(stream, comp, offs, b, c, m, n, k, ws, split_k);
     if (rc || split_k == 1)
         return rc;
-    return flashllm_hip_launch_reduce(stream, c, ws, static_cast<long>(m) * n, split_k, 0);
+    return reduce_slabs(stream, c, ws, m, n, split_k, 0);
 }
 
 int flashllm_device_tile_offsets(void* stream, const void* a, int m, int k, int* offs, long long* nnz_padded)
@@ -199,7 +208,7 @@ int flashllm_decoder_layer_linears(void*                         stream,
     rc = flashllm_spmm_partials(stream, f1.nz_weights, f1.tile_offsets, attn_out, ffn_mid, f1.m, tokens, f1.k, ws, s1);
     if (rc)
         return rc;
-    rc = s1 > 1 ? flashllm_hip_launch_reduce(stream, ffn_mid, ws, static_cast<long>(f1.m) * tokens, s1, 1)
+    rc = s1 > 1 ? reduce_slabs(stream, ffn_mid, ws, f1.m, tokens, s1, 1)
                 : flashllm_hip_launch_relu(stream, ffn_mid, static_cast<long>(f1.m) * tokens);
     if (rc)
         return rc;

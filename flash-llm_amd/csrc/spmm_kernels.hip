@@ -35,8 +35,17 @@
 // The operand exchanges are inline assembly (the compiler has no 16-byte LDS
 // exchange), followed by an explicit lgkmcnt(0).
 //
-// splitk_reduce_kernel: the separate reduction over fp16 slabs
-// (reference csrc/Reduction_Kernel.cuh:24-45), 8 bytes per lane per slab, eight slabs in flight.
+// Placement.  The GPU has eight accelerator dies (XCDs), each with its own L2, and hands the
+// workgroups of a launch to them round-robin in launch order: workgroup w runs on XCD w % 8.  The
+// SpMM kernel therefore gives the Split_K slices of one (row tile, column group) unit to workgroups
+// eight apart, and each XCD a contiguous block of units: the slabs of a unit all land in one L2.
+//
+// splitk_reduce_block_kernel: the separate reduction over fp16 slabs (reference
+// csrc/Reduction_Kernel.cuh:24-45), one workgroup per 128 x 16 block of C, given to the XCD whose L2
+// holds that block's slabs (the lines survive the kernel boundary), 16 bytes per lane per slab, eight
+// slabs in flight.  Where a workgroup runs only decides where its loads hit; the sums do not depend on it.
+// splitk_reduce_kernel: the same sums over a flat M*N range, for outputs the block kernel's layout does
+// not cover.
 #include "spmm_launch.h"
 
 #include <hip/hip_runtime.h>
@@ -54,6 +63,24 @@ constexpr int kTileCols  = 64;
 constexpr int kTileHalfs = kTileRows * kTileCols;
 constexpr int kLanes     = 64;
 constexpr int kNoTile    = 0x7fffffff;
+constexpr int kXcds      = 8;  // accelerator dies of an MI355X, each with its own L2
+
+// Workgroup w of a launch -> (unit, part), part in [0, parts): the parts of one unit go to workgroups
+// kXcds apart (one XCD under round-robin hand-out), XCD x takes the units x*per_xcd .. (x+1)*per_xcd-1;
+// units beyond a multiple of kXcds are laid out plainly behind them.
+__device__ __forceinline__ void unit_of_workgroup(unsigned w, unsigned units, unsigned parts, int& unit, int& part)
+{
+    const unsigned per_xcd = units / kXcds;
+    if (w < per_xcd * kXcds * parts) {
+        const unsigned j = w / kXcds;
+        unit             = static_cast<int>((w % kXcds) * per_xcd + j / parts);
+        part             = static_cast<int>(j % parts);
+    }
+    else {
+        unit = static_cast<int>(w / parts);
+        part = static_cast<int>(w % parts);
+    }
+}
 
 __device__ __forceinline__ void clear_tile(uint16_t* tile, int lane)
 {
@@ -112,17 +139,21 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                                                             int M,
                                                             int N,
                                                             int K,
-                                                            int split_k)
+                                                            int split_k,
+                                                            int col_groups)
 {
     __shared__ __attribute__((aligned(16))) uint16_t tile[kTileHalfs];
 
-    const int lane    = threadIdx.x;
-    const int r16     = lane & 15;  // row inside a 16-row block / output column
-    const int g       = lane >> 4;  // which 8-wide k chunk of a 32-wide k step
-    const int kt      = K / kTileCols;
-    const int slice   = blockIdx.x % split_k;
-    const int rowtile = blockIdx.x / split_k;
-    const int col0    = blockIdx.y * (16 * NB);
+    const int lane = threadIdx.x;
+    const int r16  = lane & 15;  // row inside a 16-row block / output column
+    const int g    = lane >> 4;  // which 8-wide k chunk of a 32-wide k step
+    const int kt   = K / kTileCols;
+    // unit = (row tile, column group), column group fastest: the column groups of a row tile read the
+    // same weights and meet in one L2
+    int unit, slice;
+    unit_of_workgroup(blockIdx.x, gridDim.x / split_k, split_k, unit, slice);
+    const int rowtile = unit / col_groups;
+    const int col0    = (unit % col_groups) * (16 * NB);
     // HW_ID.wave_id: which of the SIMD's wave slots this wave sits in (bit 0 tells the two apart)
     const int wave_slot = __builtin_amdgcn_s_getreg(4 | (0 << 6) | (3 << 11)) & 1;
 
@@ -346,6 +377,57 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(uint2* __restrict__ 
     c[i] = __builtin_bit_cast(uint2, h);
 }
 
+// The same sums for the output of spmm_stream_kernel, one workgroup per 128-row x 16-column block of C:
+// lane = (column, 16-byte piece of the column's 128 rows).  blocks_per_unit: 16-column blocks of one unit
+// of the SpMM kernel (its NB); the workgroup order mirrors that kernel's, so a block is summed on the XCD
+// that stored its slabs.
+template<bool RELU>
+__global__ __launch_bounds__(256) void splitk_reduce_block_kernel(_Float16* __restrict__ c,
+                                                                 const _Float16* __restrict__ ws,
+                                                                 int M,
+                                                                 int N,
+                                                                 int split_k,
+                                                                 int blocks_per_unit,
+                                                                 int col_groups)
+{
+    int unit, sub;
+    unit_of_workgroup(blockIdx.x, gridDim.x / blocks_per_unit, blocks_per_unit, unit, sub);
+    const int rowtile = unit / col_groups;
+    const int n       = ((unit % col_groups) * blocks_per_unit + sub) * 16 + (threadIdx.x >> 4);
+    if (n >= N)  // N == 8: half a block
+        return;
+    const size_t slab = static_cast<size_t>(M) * N;
+    const size_t at   = static_cast<size_t>(n) * M + static_cast<size_t>(rowtile) * kTileRows + (threadIdx.x & 15) * 8;
+    float        s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < split_k; k0 += 8) {
+        uint4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (k0 + j < split_k)
+                v[j] = *reinterpret_cast<const uint4*>(ws + (k0 + j) * slab + at);
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (k0 + j < split_k) {
+                const half8 h = __builtin_bit_cast(half8, v[j]);
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+                    s[e] += static_cast<float>(h[e]);
+            }
+    }
+    half8 h;
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+        h[e] = static_cast<_Float16>(RELU && !(s[e] > 0.f) ? 0.f : s[e]);
+    *reinterpret_cast<uint4*>(c + at) = __builtin_bit_cast(uint4, h);
+}
+
+// out[w] = id of the XCD that workgroup w of this launch ran on
+__global__ __launch_bounds__(kLanes) void xcd_probe_kernel(unsigned* __restrict__ out)
+{
+    if (threadIdx.x == 0)
+        out[blockIdx.x] = __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11));  // XCC_ID, bits 3:0
+}
+
 __global__ __launch_bounds__(256) void relu_kernel(uint4* __restrict__ x, long n8)
 {
     const long i = static_cast<long>(blockIdx.x) * 256 + threadIdx.x;
@@ -370,7 +452,7 @@ __global__ __launch_bounds__(256) void take_rows_kernel(uint4* __restrict__ dst,
 template<int NB, int DEPTH>
 int launch_spmm(hipStream_t stream, const void* comp, const int* offs, const void* b, void* out, int m, int n, int k, int split_k, int col_groups)
 {
-    const dim3 grid(static_cast<unsigned>(m / kTileRows) * split_k, col_groups, 1);
+    const dim3 grid(static_cast<unsigned>(m / kTileRows) * col_groups * split_k, 1, 1);
     hipLaunchKernelGGL((spmm_stream_kernel<NB, DEPTH>),
                        grid,
                        dim3(kLanes),
@@ -383,7 +465,8 @@ int launch_spmm(hipStream_t stream, const void* comp, const int* offs, const voi
                        m,
                        n,
                        k,
-                       split_k);
+                       split_k,
+                       col_groups);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -411,6 +494,28 @@ extern "C" int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws,
         hipLaunchKernelGGL(splitk_reduce_kernel<true>, grid, dim3(256), 0, s, cp, wp, n4, split_k);
     else
         hipLaunchKernelGGL(splitk_reduce_kernel<false>, grid, dim3(256), 0, s, cp, wp, n4, split_k);
+    return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int flashllm_hip_launch_reduce_blocks(void* stream, void* c, const void* ws, int m, int n, int split_k, int relu)
+{
+    // the units of flashllm_hip_launch_spmm for this N: 16*nb columns wide
+    const int   nb         = n <= 16 ? 1 : (n == 32 ? 2 : 4);
+    const int   col_groups = n <= 64 ? 1 : n / 64;
+    const dim3  grid(static_cast<unsigned>(m / kTileRows) * col_groups * nb);
+    hipStream_t s  = static_cast<hipStream_t>(stream);
+    _Float16*   cp = static_cast<_Float16*>(c);
+    const _Float16* wp = static_cast<const _Float16*>(ws);
+    if (relu)
+        hipLaunchKernelGGL(splitk_reduce_block_kernel<true>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, nb, col_groups);
+    else
+        hipLaunchKernelGGL(splitk_reduce_block_kernel<false>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, nb, col_groups);
+    return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int flashllm_hip_launch_xcd_probe(void* stream, unsigned* out, int workgroups)
+{
+    hipLaunchKernelGGL(xcd_probe_kernel, dim3(workgroups), dim3(kLanes), 0, static_cast<hipStream_t>(stream), out);
     return static_cast<int>(hipGetLastError());
 }
 

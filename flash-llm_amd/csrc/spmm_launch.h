@@ -23,6 +23,14 @@ int flashllm_hip_launch_spmm(void*       stream,
 // c[e] = rn16(sum_s float(ws[s*mn + e])), through max(., 0) first when relu != 0; requires mn % 4 == 0.
 int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws, long mn, int split_k, int relu);
 
+// The same sums for the slabs flashllm_hip_launch_spmm left for this (m, n): one workgroup per 128 x 16 block
+// of C, on the XCD whose L2 holds the block's slabs.  Requires M % 128 == 0, N as above, c and ws 16-byte aligned.
+int flashllm_hip_launch_reduce_blocks(void* stream, void* c, const void* ws, int m, int n, int split_k, int relu);
+
+// out[w] = id of the XCD workgroup w ran on, for a launch of `workgroups` one-wave workgroups: shows whether
+// the round-robin hand-out the placement above counts on holds on this machine.
+int flashllm_hip_launch_xcd_probe(void* stream, unsigned* out, int workgroups);
+
 // x[i] = max(x[i], 0) over n halfs (n % 8 == 0): the activation between FFN1 and FFN2.
 int flashllm_hip_launch_relu(void* stream, void* x, long n);
 

@@ -131,6 +131,22 @@ def gen_sparse_matrix_bin_file(dense, m, k, nz, offsets, sizes):
         raise CompressError(rc)
 
 
+def xcd_of_workgroups(workgroups, stream=None):
+    """XCD id of every workgroup of a launch of `workgroups` one-wave workgroups (numpy uint32 array).
+    The SpMM kernel's placement counts on ids repeating with period 8 (round-robin hand-out)."""
+    import torch
+
+    out = torch.empty(workgroups, dtype=torch.int32, device="cuda")
+    fn = lib().flashllm_hip_launch_xcd_probe
+    fn.restype = ctypes.c_int
+    fn.argtypes = [_vp, _vp, ctypes.c_int]
+    rc = fn(_stream(stream), _ptr(out), workgroups)
+    if rc:
+        raise HipError(rc)
+    torch.cuda.synchronize()
+    return out.cpu().numpy().view(np.uint32) & 15
+
+
 def _ptr(t):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
 

@@ -135,7 +135,9 @@ def test_split_k_reduction_bit_exact(product, oracle, torch_gpu):
     torch = torch_gpu
     say("reduction kernel")
     rng = np.random.default_rng(2)
-    for m, n, s in [(128, 8, 2), (1024, 16, 7), (256, 64, 32), (384, 8, 5)]:
+    # the last two shapes are outside the SpMM kernel's (M % 128, N) grid: the flat kernel sums those
+    for m, n, s in [(128, 8, 2), (1024, 16, 7), (256, 64, 32), (384, 8, 5), (2048, 32, 9), (1024, 128, 3), (256, 256, 11),
+                    (100, 8, 3), (128, 20, 6)]:
         ws_h = (rng.standard_normal((s, n * m)) * 3).astype(np.float16)
         ws = torch.from_numpy(ws_h).cuda()
         c = torch.zeros(n * m, dtype=torch.float16, device="cuda")
@@ -143,6 +145,18 @@ def test_split_k_reduction_bit_exact(product, oracle, torch_gpu):
         torch.cuda.synchronize()
         want = oracle.splitk_reduce(ws_h, n * m, s)
         assert np.array_equal(c.cpu().numpy().view(np.uint16), want.view(np.uint16))
+
+
+def test_workgroups_go_round_robin_over_the_xcds(product, torch_gpu):
+    """The placement of slices and of the reduction's workgroups counts on workgroup w running on XCD w % 8.
+    Results never depend on it (the reduction is a separate kernel), only where its loads hit."""
+    say("xcd probe")
+    ids = product.xcd_of_workgroups(2016)
+    assert ids.max() < 8
+    distinct = len(set(ids.tolist()))
+    same_as_first_round = float(np.mean(ids == ids[np.arange(ids.size) % 8]))
+    say(f"  {distinct} XCD ids; share of workgroups on the XCD of workgroup w % 8: {same_as_first_round:.3f}")
+    assert distinct in (1, 2, 4, 8)  # whole GPU, or one of its partition modes
 
 
 def test_partials_then_reduce_equals_api(product, oracle, torch_gpu):

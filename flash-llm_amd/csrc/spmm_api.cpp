@@ -89,6 +89,39 @@ int flashllm_spmm_splitk(void*       stream,
     return reduce_slabs(stream, c, ws, m, n, split_k, 0);
 }
 
+// SpMM_SplitK_API for callers that must not allocate and hold no workspace: the slabs go to the
+// library's fixed device array.
+int flashllm_spmm_splitk_static(void*       stream,
+                                const void* a,
+                                const void* comp,
+                                const int*  offs,
+                                const void* b,
+                                void*       c,
+                                int         m,
+                                int         n,
+                                int         k,
+                                int         split_k)
+{
+    void* ws = nullptr;
+    if (split_k > 1) {
+        // sizes first: no launch and no symbol lookup for a call that cannot fit
+        if (m <= 0 || n <= 0)
+            return hipErrorInvalidValue;
+        const size_t need = flashllm_workspace_bytes(m, n, split_k);
+        if (need > FLASHLLM_STATIC_WORKSPACE_BYTES) {
+            std::fprintf(stderr,
+                         "flashllm_spmm_splitk_static: Split_K*M*N*2 = %zu bytes exceeds the library's fixed slab storage of %u bytes; "
+                         "use a smaller Split_K or flashllm_spmm_splitk with a workspace of your own\n",
+                         need, FLASHLLM_STATIC_WORKSPACE_BYTES);
+            return hipErrorInvalidValue;
+        }
+        const int rc = flashllm_hip_static_workspace(&ws);
+        if (rc)
+            return rc;
+    }
+    return flashllm_spmm_splitk(stream, a, comp, offs, b, c, m, n, k, ws, split_k);
+}
+
 int flashllm_device_tile_offsets(void* stream, const void* a, int m, int k, int* offs, long long* nnz_padded)
 {
     if (!a || !offs || (reinterpret_cast<uintptr_t>(a) & 15u))

@@ -51,6 +51,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace {
 
 using half8   = _Float16 __attribute__((ext_vector_type(8)));
@@ -470,7 +472,37 @@ int launch_spmm(hipStream_t stream, const void* comp, const int* offs, const voi
     return static_cast<int>(hipGetLastError());
 }
 
+constexpr int      kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
 }  // namespace
+
+// Library-owned slab storage for callers that cannot provide (or allocate) a Reduction_Workspace: a fixed
+// array in the code object's own device memory, one copy per GPU the library runs on, held until the
+// process ends.  In host code the array's name is only a handle: the device address comes from
+// hipGetSymbolAddress, once per device, and that pointer is what kernels receive.
+static __device__ __align__(256) unsigned char scratch[FLASHLLM_STATIC_WORKSPACE_BYTES];
+
+extern "C" int flashllm_hip_static_workspace(void** ptr)
+{
+    int        dev = -1;
+    hipError_t e   = hipGetDevice(&dev);
+    if (e != hipSuccess)
+        return static_cast<int>(e);
+    if (dev < 0 || dev >= kMaxDevices)
+        return static_cast<int>(hipErrorInvalidDevice);
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {  // first call on this device (two threads racing here resolve the same address)
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess)
+            return static_cast<int>(e);
+        if (!p)
+            return static_cast<int>(hipErrorInvalidSymbol);
+        g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    *ptr = p;
+    return 0;
+}
 
 extern "C" int flashllm_hip_launch_spmm(
     void* stream, const void* comp, const int* offs, const void* b, void* out, int m, int n, int k, int split_k)

@@ -4,9 +4,16 @@
 #ifndef FLASHLLM_AMD_SPMM_LAUNCH_H
 #define FLASHLLM_AMD_SPMM_LAUNCH_H
 
+// size of the library-owned slab storage behind flashllm_hip_static_workspace
+#define FLASHLLM_STATIC_WORKSPACE_BYTES (32u << 20)
+
 #ifdef __cplusplus
 extern "C" {
 #endif
+
+// *ptr = device address, on the current device, of the library's own fixed slab storage
+// (FLASHLLM_STATIC_WORKSPACE_BYTES, 256-byte aligned).  Resolved once per device; allocates nothing.
+int flashllm_hip_static_workspace(void** ptr);
 
 // out: C when split_k == 1, else the slab workspace (split_k * M * N halfs).
 // Requires M % 128 == 0, K % 64 == 0, N in {8,16,32,64} or N % 64 == 0.

@@ -42,6 +42,7 @@ SIGNATURES = {
     "flashllm_free": (None, [_vp]),
     "flashllm_set_compress_threads": (None, [ctypes.c_int]),
     "flashllm_spmm_splitk": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int]),
+    "flashllm_spmm_splitk_static": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "flashllm_spmm_partials": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int]),
     "flashllm_splitk_reduce": (ctypes.c_int, [_vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "flashllm_device_tile_offsets": (ctypes.c_int, [_vp, _vp, ctypes.c_int, ctypes.c_int, _vp, ctypes.POINTER(ctypes.c_longlong)]),
@@ -168,6 +169,16 @@ def spmm_splitk(comp, offs, b, c, m, n, k, workspace, split_k, stream=None, a=No
     """SpMM_SplitK_API on torch device tensors; asynchronous on `stream`
     (default: torch's current stream).  Raises HipError on a non-zero code."""
     rc = lib().flashllm_spmm_splitk(_stream(stream), _ptr(a), _ptr(comp), _ptr(offs), _ptr(b), _ptr(c), m, n, k, _ptr(workspace), split_k)
+    if rc:
+        raise HipError(rc)
+
+
+STATIC_WORKSPACE_MAX_BYTES = 32 << 20
+
+
+def spmm_splitk_static(comp, offs, b, c, m, n, k, split_k, stream=None):
+    """flashllm_spmm_splitk_static: the slabs live in the library's own fixed device array."""
+    rc = lib().flashllm_spmm_splitk_static(_stream(stream), None, _ptr(comp), _ptr(offs), _ptr(b), _ptr(c), m, n, k, split_k)
     if rc:
         raise HipError(rc)
 

@@ -60,6 +60,29 @@ int flashllm_spmm_splitk(void*       stream,
                          int         Split_K);
 
 /*
+ * flashllm_spmm_splitk without the Reduction_Workspace argument, for callers that cannot allocate
+ * device memory and hold no workspace (code under stream capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  It has no counterpart in the reference.  The Split_K slabs go to a fixed
+ * array of FLASHLLM_STATIC_WORKSPACE_MAX_BYTES that is part of the library's device image (every GPU
+ * the library runs on holds one copy until the process ends); the call allocates and frees nothing.
+ * Split_K * M * N * 2 bytes beyond that size are rejected with hipErrorInvalidValue (1) and a message
+ * on stderr, before anything is launched.  All calls on one GPU share the array: calls that overlap
+ * on one GPU (different streams or threads) race on the slabs; calls on one stream are ordered and safe.
+ * Every slab is fully written before it is read, so nothing needs clearing between calls.
+ */
+#define FLASHLLM_STATIC_WORKSPACE_MAX_BYTES (32u << 20)
+int flashllm_spmm_splitk_static(void*       stream,
+                                const void* A,
+                                const void* Compressed_A,
+                                const int*  TileOffsets,
+                                const void* B,
+                                void*       C,
+                                int         M,
+                                int         N,
+                                int         K,
+                                int         Split_K);
+
+/*
  * The first half of flashllm_spmm_splitk alone (reference
  * csrc/SpMM_API.cu:73-118): launches only the SpMM kernel and leaves the
  * Split_K fp16 slabs in Reduction_Workspace (or writes C when Split_K == 1).

@@ -159,35 +159,33 @@ size_t flashllm_workspace_bytes(int m, int n, int split_k)
     return static_cast<size_t>(split_k) * m * n * sizeof(uint16_t);
 }
 
-// One wave streams one (row tile, K slice, column group).  Two waves per SIMD, 8 per CU, is what the
-// kernel is tuned for and what its registers allow at N >= 32; at N <= 16 a CU could hold 10 (16 KB LDS
-// tiles), but a ninth wave per CU already measures 5 % slower.  The grid should fill those slots on
-// all 256 CUs exactly once, in slices of equal length: a second round of workgroups would run at a
-// fraction of the occupancy.
+// One wave streams one (row tile, K slice, column group); a CU holds eight of them (two per SIMD, what the
+// registers allow at N >= 32), so 2048 fit at once and a grid beyond that runs a second, mostly empty round
+// (36864x9216, N = 32: 56 us at 7 slices = 2016 waves, 74 us at 8).  Among the Split_K values of one round the
+// time follows
+//     longest slice (k tiles) x (2 + resident waves per CU)  +  Split_K x (0.5 + 0.5 x (N/16) x (M/36864)):
+// a wave needs a fixed time per tile plus what its neighbours on the CU take from it (LDS and issue slots
+// are shared), so more slices only help while they shorten the longest slice faster than they crowd the CU
+// (12288x12288: 16 slices of 12 tiles beat 20 slices of which the last has 2); every slab costs a write and
+// a read of M*N halfs and a step of the reduction.  Constants fitted to the whole-call times of the
+// reference's twelve weight shapes (kernel_benchmark/benchmark.sh:13-14) x N in {8,16,32,64} at 80 %
+// sparsity: mean 0.3 % and at most 4.6 % above the best Split_K of each case.
 int flashllm_splitk_heuristic(int m, int n, int k)
 {
     if (m <= 0 || k <= 0 || n <= 0 || m % 128 || k % 64)
         return 1;
-    const int  kt         = k / 64;
-    const int  col_groups = n <= 64 ? 1 : n / 64;
-    const long units      = static_cast<long>(m / 128) * col_groups;
-    const long slots      = 256L * 8;
-    // Largest split that still runs in one round; a second round would run at a fraction of the
-    // occupancy (measured at 36864x9216, N=16: 46 us at 7 slices = 2016 waves, 49 us at 8, 62 us at 9).
-    long s_max = slots / units;
-    if (s_max > 32)
-        s_max = 32;  // workspace sizes in existing callers assume at most 32 slabs
-    if (s_max > kt)
-        s_max = kt;
-    if (s_max < 1)
-        s_max = 1;
-    // Time follows the longest slice (in k tiles); each slab adds a write and a read of M*N halfs
-    // and a little reduction time, about a quarter of a k tile's worth.
-    int    best      = 1;
-    double best_cost = 1e30;
-    for (int s = 1; s <= s_max; s++) {
-        const int    avg  = (kt - 1) / s + 1;
-        const double cost = avg + (s > 1 ? 0.25 * s : 0.0);
+    const int    kt         = k / 64;
+    const int    col_groups = n <= 64 ? 1 : n / 64;
+    const long   units      = static_cast<long>(m / 128) * col_groups;
+    const long   slots      = 256L * 8;
+    const double per_slab   = 0.5 + 0.5 * (n / 16.0) * (m / 36864.0);
+    int          best       = 1;
+    double       best_cost  = 1e30;
+    for (int s = 1; s <= 32 && s <= kt; s++) {  // workspace sizes in existing callers assume at most 32 slabs
+        if (s > 1 && units * s > slots)
+            break;
+        const int    longest = (kt - 1) / s + 1;
+        const double cost    = longest * (2.0 + units * s / 256.0) + (s > 1 ? s * per_slab : 0.0);
         if (cost < best_cost) {
             best_cost = cost;
             best      = s;

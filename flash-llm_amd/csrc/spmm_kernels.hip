@@ -33,7 +33,7 @@
 // (global_load_lds_dwordx4) measured the same at N <= 32 and slower at
 // N = 64, where its 8 KB per wave cost two resident waves per CU.
 // The operand exchanges are inline assembly (the compiler has no 16-byte LDS
-// exchange), followed by an explicit lgkmcnt(0).
+// exchange) and carry their own lgkmcnt(0) inside the same statement.
 //
 // Placement.  The GPU has eight accelerator dies (XCDs), each with its own L2, and hands the
 // workgroups of a launch to them round-robin in launch order: workgroup w runs on XCD w % 8.  The
@@ -119,15 +119,63 @@ __device__ __forceinline__ uint32_t lds_offset(const void* p)
     return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) void*)(p)));
 }
 
-// Returns the 16 bytes at lds_byte_addr and stores zeros there, one LDS instruction.  The result is
-// valid after the next s_waitcnt lgkmcnt(0).
-__device__ __forceinline__ uintx4 take_and_clear_16(uint32_t lds_byte_addr)
+// Takes eight 16-byte operands out of LDS (one per 16-row block, at addr[0..7]) and leaves zeros behind:
+// ds_wrxchg2_rtn_b64 returns the operand and stores the zeros in one LDS instruction.  The compiler does not
+// track the LDS returns of inline assembly, so the exchanges and the wait for them sit in ONE statement, with
+// early-clobber outputs: no register of a[] can be read, moved or spilled while its exchange is in flight.
+using uintx2 = uint32_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void take_8_and_wait(uintx4 (&a)[8], const uint32_t (&addr)[8])
 {
-    using uintx2 = uint32_t __attribute__((ext_vector_type(2)));
     const uintx2 zero = {0u, 0u};
-    uintx4       old;
-    asm volatile("ds_wrxchg2_rtn_b64 %0, %1, %2, %2 offset1:1" : "=v"(old) : "v"(lds_byte_addr), "v"(zero) : "memory");
-    return old;
+    asm volatile(
+        "ds_wrxchg2_rtn_b64 %0, %8, %16, %16 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %1, %9, %16, %16 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %2, %10, %16, %16 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %3, %11, %16, %16 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %4, %12, %16, %16 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %5, %13, %16, %16 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %6, %14, %16, %16 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %7, %15, %16, %16 offset1:1\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(a[0]), "=&v"(a[1]), "=&v"(a[2]), "=&v"(a[3]), "=&v"(a[4]), "=&v"(a[5]), "=&v"(a[6]), "=&v"(a[7])
+        : "v"(addr[0]), "v"(addr[1]), "v"(addr[2]), "v"(addr[3]), "v"(addr[4]), "v"(addr[5]), "v"(addr[6]), "v"(addr[7]), "v"(zero)
+        : "memory");
+}
+
+// Sixteen operands (both 32-wide k steps): all sixteen exchanges are issued back to back, then one wait.
+// Two statements, because one statement takes at most thirty operands: the first issues eight exchanges,
+// the second, directly behind it, the other eight and the wait, and carries the first eight as in/out
+// operands so that they cannot be used before that wait.
+__device__ __forceinline__ void take_16_and_wait(uintx4 (&a0)[8], uintx4 (&a1)[8], const uint32_t (&addr0)[8], const uint32_t (&addr1)[8])
+{
+    const uintx2 zero = {0u, 0u};
+    asm volatile(
+        "ds_wrxchg2_rtn_b64 %0, %8, %16, %16 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %1, %9, %16, %16 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %2, %10, %16, %16 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %3, %11, %16, %16 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %4, %12, %16, %16 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %5, %13, %16, %16 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %6, %14, %16, %16 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %7, %15, %16, %16 offset1:1"
+        : "=&v"(a0[0]), "=&v"(a0[1]), "=&v"(a0[2]), "=&v"(a0[3]), "=&v"(a0[4]), "=&v"(a0[5]), "=&v"(a0[6]), "=&v"(a0[7])
+        : "v"(addr0[0]), "v"(addr0[1]), "v"(addr0[2]), "v"(addr0[3]), "v"(addr0[4]), "v"(addr0[5]), "v"(addr0[6]), "v"(addr0[7]), "v"(zero)
+        : "memory");
+    asm volatile(
+        "ds_wrxchg2_rtn_b64 %0, %16, %24, %24 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %1, %17, %24, %24 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %2, %18, %24, %24 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %3, %19, %24, %24 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %4, %20, %24, %24 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %5, %21, %24, %24 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %6, %22, %24, %24 offset1:1\n\t"
+        "ds_wrxchg2_rtn_b64 %7, %23, %24, %24 offset1:1\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(a1[0]), "=&v"(a1[1]), "=&v"(a1[2]), "=&v"(a1[3]), "=&v"(a1[4]), "=&v"(a1[5]), "=&v"(a1[6]), "=&v"(a1[7]),
+          "+v"(a0[0]), "+v"(a0[1]), "+v"(a0[2]), "+v"(a0[3]), "+v"(a0[4]), "+v"(a0[5]), "+v"(a0[6]), "+v"(a0[7])
+        : "v"(addr1[0]), "v"(addr1[1]), "v"(addr1[2]), "v"(addr1[3]), "v"(addr1[4]), "v"(addr1[5]), "v"(addr1[6]), "v"(addr1[7]), "v"(zero)
+        : "memory");
 }
 
 // NB: 16-column blocks per wave (1 for N <= 16, 2 for N = 32, 4 for N >= 64).
@@ -189,6 +237,12 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
             bptr[nb] = B + static_cast<size_t>(n) * K + g * 8;
         }
         const uint32_t tile_lds = lds_offset(&tile[0]);
+        uint32_t       a_addr0[8], a_addr1[8];  // LDS byte addresses of this lane's operands: k step 0 / 1 of row block rb
+#pragma unroll
+        for (int rb = 0; rb < 8; rb++) {
+            a_addr0[rb] = tile_lds + rb * (16 * kTileCols * 2) + a_off0;
+            a_addr1[rb] = tile_lds + rb * (16 * kTileCols * 2) + a_off1;
+        }
         half8          bfrag[2][NB];  // B fragments of the open tile
         auto           load_b = [&](int t) {
 #pragma unroll
@@ -226,40 +280,34 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                         if (tile_hi > tile_lo) {
                             // NB <= 2: all 16 operands in one batch.  NB == 4: one 32-wide k step at a time, which
                             // keeps the kernel within 256 VGPRs (two waves per SIMD).
-                            constexpr int    kBatch = NB >= 4 ? 1 : 2;
+                            if constexpr (NB >= 4) {
 #pragma unroll
-                            for (int k0 = 0; k0 < 2; k0 += kBatch) {
-                                uintx4 a[kBatch][8];
-#pragma unroll
-                                for (int ks = 0; ks < kBatch; ks++)
-#pragma unroll
-                                    for (int rb = 0; rb < 8; rb++)
-                                        a[ks][rb] = take_and_clear_16(tile_lds + rb * (16 * kTileCols * 2) +
-                                                                      ((k0 + ks) ? a_off1 : a_off0));
-                                // the exchanges above have landed
-                                if constexpr (kBatch == 2)
-                                    asm volatile("s_waitcnt lgkmcnt(0)"
-                                                 : "+v"(a[0][0]), "+v"(a[0][1]), "+v"(a[0][2]), "+v"(a[0][3]),
-                                                   "+v"(a[0][4]), "+v"(a[0][5]), "+v"(a[0][6]), "+v"(a[0][7]),
-                                                   "+v"(a[kBatch - 1][0]), "+v"(a[kBatch - 1][1]), "+v"(a[kBatch - 1][2]),
-                                                   "+v"(a[kBatch - 1][3]), "+v"(a[kBatch - 1][4]), "+v"(a[kBatch - 1][5]),
-                                                   "+v"(a[kBatch - 1][6]), "+v"(a[kBatch - 1][7])
-                                                 :
-                                                 : "memory");
-                                else
-                                    asm volatile("s_waitcnt lgkmcnt(0)"
-                                                 : "+v"(a[0][0]), "+v"(a[0][1]), "+v"(a[0][2]), "+v"(a[0][3]),
-                                                   "+v"(a[0][4]), "+v"(a[0][5]), "+v"(a[0][6]), "+v"(a[0][7])
-                                                 :
-                                                 : "memory");
-#pragma unroll
-                                for (int ks = 0; ks < kBatch; ks++)
+                                for (int ks = 0; ks < 2; ks++) {
+                                    uintx4 a[8];
+                                    take_8_and_wait(a, ks ? a_addr1 : a_addr0);
 #pragma unroll
                                     for (int rb = 0; rb < 8; rb++)
 #pragma unroll
                                         for (int nb = 0; nb < NB; nb++)
                                             acc[nb][rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                                __builtin_bit_cast(half8, a[ks][rb]), bfrag[k0 + ks][nb], acc[nb][rb], 0, 0, 0);
+                                                __builtin_bit_cast(half8, a[rb]), bfrag[ks][nb], acc[nb][rb], 0, 0, 0);
+                                }
+                            }
+                            else {
+                                uintx4 a0[8], a1[8];
+                                take_16_and_wait(a0, a1, a_addr0, a_addr1);
+#pragma unroll
+                                for (int rb = 0; rb < 8; rb++)
+#pragma unroll
+                                    for (int nb = 0; nb < NB; nb++)
+                                        acc[nb][rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                            __builtin_bit_cast(half8, a0[rb]), bfrag[0][nb], acc[nb][rb], 0, 0, 0);
+#pragma unroll
+                                for (int rb = 0; rb < 8; rb++)
+#pragma unroll
+                                    for (int nb = 0; nb < NB; nb++)
+                                        acc[nb][rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                            __builtin_bit_cast(half8, a1[rb]), bfrag[1][nb], acc[nb][rb], 0, 0, 0);
                             }
                         }
                         t++;

@@ -221,6 +221,10 @@ __global__ __launch_bounds__(kLanes* kEncodeWaves) void encode_tiles_kernel(cons
     __syncthreads();
 
     uint32_t* out_tile = out + static_cast<size_t>(offs[t]) * 4;
+    // Never write outside this tile's range of Compressed_A, whatever TileOffsets says: with offsets that were
+    // not computed from this very matrix the output is meaningless, but it stays inside the caller's buffer.
+    const int room = (offs[t + 1] - offs[t]) * 4;
+    count          = count < room ? count : room;
     auto      emit     = [&](int b, int h, uint32_t item) {
         const int j = above[h] + __builtin_popcount(reach[h] & ((1u << b) - 1u));
         int       d;

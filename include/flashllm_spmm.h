@@ -115,8 +115,8 @@ int flashllm_splitk_heuristic(int M, int N, int K);
  * Tiled-CSL compression on the GPU for a dense matrix that is already in
  * device memory: the bytes of flashllm_init_sparse_matrix_a (reference
  * InitSparseMatrixA_API, csrc/SpMM_API.cu:163-360, which runs on the host on
- * one thread), produced by one wave per 128x64 tile.  Two calls, because the
- * caller owns the output allocation:
+ * one thread), produced by one workgroup of four waves per 128x64 tile.  Two
+ * calls, because the caller owns the output allocation:
  *
  *  flashllm_device_tile_offsets fills TileOffsets (device, (M/128)*(K/64)+2
  *  ints) and, when NNZ_padded is not NULL, waits for the stream and stores the
@@ -128,7 +128,12 @@ int flashllm_splitk_heuristic(int M, int N, int K);
  *
  * A: device pointer, row-major M x K halfs, 16-byte aligned; M % 128 == 0,
  * K % 64 == 0.  Returns 0, a negative FLASHLLM_E_* code or a positive
- * hipError_t value.
+ * hipError_t value.  TileOffsets given to flashllm_device_compress must be
+ * what flashllm_device_tile_offsets computed for this very A: the encoder
+ * trusts them for where each tile goes.  With other offsets the contents of
+ * Compressed_A are unspecified; the encoder still never writes outside
+ * [TileOffsets[t], TileOffsets[t+1]) for tile t, and there is no error code
+ * for it (the call is asynchronous).
  */
 int flashllm_device_tile_offsets(void* stream, const void* A, int M, int K, int* TileOffsets, long long* NNZ_padded);
 int flashllm_device_compress(void* stream, const void* A, int M, int K, const int* TileOffsets, void* Compressed_A);

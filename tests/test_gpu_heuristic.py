@@ -1,0 +1,60 @@
+"""The Split_K the library recommends (flashllm_splitk_heuristic, which stands in for the reference's per-shape
+tables hand-tuned for A100, kernel_benchmark/benchmark.sh:13-15) against its neighbours on the five benchmark shapes:
+the whole SpMM_SplitK_API call at the recommended value may take at most 5 % longer than at the best of
+{s-2 .. s+2}.  Weights are pruned and compressed on the GPU; every timed loop rotates over enough copies of
+Compressed_A that the weights come from HBM; each figure is the median of three loops."""
+import sys
+import time
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(36864, 9216, 16), (9216, 36864, 16), (9216, 9216, 16), (36864, 12288, 32), (49152, 12288, 32)]
+
+
+def median_time_us(torch, fn, loops=3, steps=150, settle_s=0.1):
+    t0 = time.perf_counter()
+    i = 0
+    while time.perf_counter() - t0 < settle_s:
+        for _ in range(50):
+            fn(i)
+            i += 1
+        torch.cuda.synchronize()
+    out = []
+    for _ in range(loops):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(steps):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        out.append(e0.elapsed_time(e1) / steps * 1e3)
+    return sorted(out)[loops // 2]
+
+
+@pytest.mark.parametrize("m,k,n", SHAPES)
+def test_recommended_split_k_is_within_5_percent_of_its_neighbours(product, m, k, n):
+    import torch
+
+    assert torch.cuda.is_available()
+    print(f"split_k neighbourhood {m}x{k} N={n}", flush=True)
+    sys.stdout.flush()
+    g = torch.Generator(device="cuda").manual_seed(m + k + n)
+    a = torch.randn(m, k, dtype=torch.float16, device="cuda", generator=g) * 0.02
+    a = torch.where(torch.rand(m, k, device="cuda", generator=g) < 0.2, a, torch.zeros((), dtype=torch.float16, device="cuda"))
+    comp, offs = product.device_compress(a)
+    del a
+    copies = max(2, min(8, int(6e8 // (4 * comp.numel())) + 1))
+    comps = [comp] + [comp.clone() for _ in range(copies - 1)]
+    b = torch.randn(n * k, dtype=torch.float16, device="cuda", generator=g)
+    c = torch.empty(n * m, dtype=torch.float16, device="cuda")
+    s = product.splitk_heuristic(m, n, k)
+    cands = [x for x in range(s - 2, s + 3) if 1 <= x <= min(32, k // 64)]
+    ws = torch.empty(max(cands) * n * m, dtype=torch.float16, device="cuda")
+    times = {}
+    for x in cands:
+        times[x] = median_time_us(torch, lambda i: product.spmm_splitk(comps[i % copies], offs, b, c, m, n, k, ws, x))
+    print("  " + "  ".join(f"{x}: {t:.2f} us" + ("*" if x == s else "") for x, t in times.items()), flush=True)
+    assert times[s] <= 1.05 * min(times.values()), (s, times)

@@ -61,6 +61,9 @@ int flashllm_spmm_partials(void*       stream,
     const int bad = check_shape(comp, offs, b, c, m, n, k, ws, split_k);
     if (bad)
         return bad;
+    // wide B: four waves share every scattered tile; otherwise one wave per (row tile, slice, column group)
+    if (n % 128 == 0)
+        return flashllm_hip_launch_spmm_group(stream, comp, offs, b, split_k == 1 ? c : ws, m, n, k, split_k);
     return flashllm_hip_launch_spmm(stream, comp, offs, b, split_k == 1 ? c : ws, m, n, k, split_k);
 }
 
@@ -174,7 +177,29 @@ int flashllm_splitk_heuristic(int m, int n, int k)
 {
     if (m <= 0 || k <= 0 || n <= 0 || m % 128 || k % 64)
         return 1;
-    const int    kt         = k / 64;
+    const int kt = k / 64;
+    if (n % 128 == 0) {
+        // Wide B goes to the four-wave kernel: a workgroup per (row tile, slice, 128 columns), up to three resident
+        // per CU (768 at once), handed out as earlier ones finish, so more than one round is no loss by itself.
+        // A workgroup alone on its CU needs 1.17 us per tile, 2.1 us when three share the CU; every slab costs
+        // a write and a read of M*N halfs (about 5 TB/s).  Fitted to 36864x9216 at N = 128 / 256.
+        const long   units     = static_cast<long>(m / 128) * (n / 128);
+        const double slab_us   = 4.0 * m * n / 5e6;
+        int          best      = 1;
+        double       best_cost = 1e30;
+        for (int s = 1; s <= 32 && s <= kt; s++) {
+            const double wgs      = static_cast<double>(units) * s;
+            const double resident = wgs / 256.0 < 3.0 ? wgs / 256.0 : 3.0;
+            const double rounds   = wgs > 768.0 ? wgs / 768.0 : 1.0;
+            const int    longest  = (kt - 1) / s + 1;
+            const double cost     = longest * (1.17 + 0.47 * (resident > 1.0 ? resident - 1.0 : 0.0)) * rounds + (s > 1 ? s * slab_us : 0.0);
+            if (cost < best_cost) {
+                best_cost = cost;
+                best      = s;
+            }
+        }
+        return best;
+    }
     const int    col_groups = n <= 64 ? 1 : n / 64;
     const long   units      = static_cast<long>(m / 128) * col_groups;
     const long   slots      = 256L * 8;

@@ -52,6 +52,7 @@
 #include <stdint.h>
 
 #include <atomic>
+#include <type_traits>
 
 namespace {
 
@@ -366,6 +367,234 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// spmm_group_kernel: the kernel for wide B (N a multiple of 128).  The one-wave kernel above pays the whole
+// cost of a tile (scatter, take it out of LDS, clear it) once per 64 output columns; here four waves share it,
+// as the reference's four warps share one A tile for its wide-N configurations (csrc/SpMM_API.cu:97-112).
+// A workgroup of four waves owns (row tile, K slice, group of 4*16*NBW columns):
+//   * all four stream and scatter: round r of a tile gives wave w the 64 vectors (r*4 + w)*64 .. of the
+//     tile's range of Compressed_A; the vectors of the next kAhead tiles are in flight per wave;
+//   * each wave multiplies the whole tile by its own 16*NBW columns: 16 plain 16-byte operand reads
+//     (no clearing: the tile has four readers), 16*NBW MFMAs, B fragments in registers;
+//   * three tile buffers rotate, so one barrier per tile is enough: in step t a wave reads tile t from one
+//     buffer (complete since the previous barrier), scatters its part of tile t+1 into the second and clears
+//     its quarter of the third (read by everybody before the previous barrier).
+// Every step issues the same number of global loads in the same order (R stream loads and 2*NBW fragment
+// loads, addresses clamped instead of skipped) and every round has all three steps, so the waits the compiler
+// places are exact counts that never drain the stream, and the accumulators stay where they are (with early
+// exits from the unrolled round the register allocation more than doubled).  A tile with more than R*256
+// vectors takes its remaining rounds on a slow path.
+constexpr int kGroupWaves   = 4;
+constexpr int kGroupThreads = kGroupWaves * kLanes;
+constexpr int kAhead        = 3;  // tiles of the stream in flight per wave = the three buffers' rotation
+
+template<int NBW, int R>
+__device__ __forceinline__ void spmm_group_body(uint16_t (&tiles)[3][kTileHalfs],
+                                                const uint4* __restrict__ comp,
+                                                const int* __restrict__ toff,
+                                                const _Float16* __restrict__ B,
+                                                _Float16* __restrict__ o,
+                                                int M,
+                                                int N,
+                                                int K,
+                                                int kb,
+                                                int ke,
+                                                int col0,
+                                                int vmax)
+{
+    const int lane = threadIdx.x & (kLanes - 1);
+    const int wave = threadIdx.x / kLanes;
+
+    floatx4 acc[NBW][8];
+#pragma unroll
+    for (int nb = 0; nb < NBW; nb++)
+#pragma unroll
+        for (int rb = 0; rb < 8; rb++)
+            acc[nb][rb] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    // column col0 + r16 of B; block nb is 16 columns (16 * K halfs) further on (N is a multiple of 128 here)
+    const _Float16* bptr = B + static_cast<size_t>(col0 + (lane & 15)) * K + (lane >> 4) * 8;
+    // operand of this lane inside a 16-row block: row r16 = lane % 16, 16-byte chunk (ks*4 + lane/16) ^ (row%8)
+    const int a_off0 = (lane & 15) * (kTileCols * 2) + (((lane >> 4) ^ (lane & 7)) << 4);
+    const int a_off1 = a_off0 ^ 64;
+
+    uint4 ring[kAhead][R];  // ring[p][r]: this wave's vectors of round r of the tile in slot p
+    int   slot_lo[kAhead], slot_n[kAhead];
+    half8 bfrag[2][NBW];
+
+    auto tile_range = [&](int t, int& lo, int& n) {  // tiles at or beyond ke are empty
+        const int a = t < ke ? t : ke, b = t + 1 < ke ? t + 1 : ke;
+        lo          = toff[a];
+        n           = toff[b] - lo;
+    };
+    int  ahead_lo, ahead_n;  // range of the tile the next request is for, fetched one request earlier
+    auto request = [&](auto pp, int t) {  // this wave's R loads of tile t into slot p, always issued
+        constexpr int p = decltype(pp)::value;
+        slot_lo[p]      = ahead_lo;
+        slot_n[p]       = ahead_n;
+        tile_range(t + 1, ahead_lo, ahead_n);  // requests go tile by tile, so the next one is for t + 1
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            int v      = slot_lo[p] + (r * kGroupWaves + wave) * kLanes + lane;
+            v          = v < vmax ? v : vmax;
+            ring[p][r] = load_stream(comp + v);
+        }
+    };
+    auto load_b = [&](int t) {  // always issued: past the end the last tile's fragments are fetched again
+        const int tc = t < ke ? t : ke - 1;
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+            for (int nb = 0; nb < NBW; nb++)
+                bfrag[ks][nb] = *reinterpret_cast<const half8*>(bptr + static_cast<size_t>(nb) * 16 * K + tc * kTileCols + ks * 32);
+    };
+    auto scatter_slot = [&](auto pp, uint16_t* buf) {
+        constexpr int p = decltype(pp)::value;
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if ((r * kGroupWaves + wave) * kLanes + lane < slot_n[p])
+                scatter_vector(buf, ring[p][r]);
+        // a tile longer than R rounds: the rest straight from memory
+        for (int r = R; r * kGroupThreads < slot_n[p]; r++) {
+            const int i = (r * kGroupWaves + wave) * kLanes + lane;
+            if (i < slot_n[p])
+                scatter_vector(buf, load_stream(comp + slot_lo[p] + i));
+        }
+    };
+    auto clear_quarter = [&](uint16_t* buf) {
+        uint4 zero = {0u, 0u, 0u, 0u};
+        asm volatile("" : "+v"(zero.x), "+v"(zero.y), "+v"(zero.z), "+v"(zero.w));  // made here, not kept in registers round the loop
+        uint4* q = reinterpret_cast<uint4*>(buf) + wave * (kTileHalfs * 2 / 16 / kGroupWaves);
+#pragma unroll
+        for (int i = 0; i < kTileHalfs * 2 / 16 / kGroupThreads; i++)
+            q[i * kLanes + lane] = zero;
+    };
+    constexpr int kAtOnce = 8;
+    auto          multiply = [&](const uint16_t* buf) {
+        const char* base = reinterpret_cast<const char*>(buf);
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+            for (int part = 0; part < 8 / kAtOnce; part++) {  // a few row blocks at a time keeps the operand registers few
+                half8 a[kAtOnce];
+#pragma unroll
+                for (int i = 0; i < kAtOnce; i++)
+                    a[i] = *reinterpret_cast<const half8*>(base + (part * kAtOnce + i) * (16 * kTileCols * 2) + (ks ? a_off1 : a_off0));
+#pragma unroll
+                for (int i = 0; i < kAtOnce; i++)
+#pragma unroll
+                    for (int nb = 0; nb < NBW; nb++)
+                        // in place (the accumulator is an in/out operand): left to itself the compiler gives the
+                        // unrolled steps accumulators of their own and runs out of registers moving between them
+                        asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc[nb][part * kAtOnce + i]) : "v"(a[i]), "v"(bfrag[ks][nb]));
+            }
+    };
+    // all LDS traffic of this wave has landed, then everybody meets: nothing here waits for global memory
+    auto meet = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+    // prologue: request kAhead tiles, clear the buffers, scatter the first tile
+    tile_range(kb, ahead_lo, ahead_n);
+    request(std::integral_constant<int, 0>{}, kb + 0);
+    request(std::integral_constant<int, 1>{}, kb + 1);
+    request(std::integral_constant<int, 2>{}, kb + 2);
+    load_b(kb);
+    clear_quarter(tiles[0]);
+    clear_quarter(tiles[1]);
+    clear_quarter(tiles[2]);
+    meet();
+    scatter_slot(std::integral_constant<int, 0>{}, tiles[0]);
+    request(std::integral_constant<int, 0>{}, kb + kAhead);
+    meet();
+
+    // step j of a round of three: tile t sits in buffer j and came from slot j.  The MFMAs go first (their
+    // operands have been complete since the last meeting) and run while the wave scatters the next tile; the
+    // next tile's fragments are requested right behind them and have the rest of the step to arrive.
+    // Rounds are always whole: a step past the slice's end finds an empty (all-zero) buffer, scatters nothing,
+    // and multiplies zeros by zeros (its fragments are blanked, so that an Inf or NaN in B cannot leak in).
+    auto step = [&](auto jj, int t) {
+        constexpr int j = decltype(jj)::value, next = (j + 1) % kAhead;
+        if (t >= ke) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                for (int nb = 0; nb < NBW; nb++)
+                    bfrag[ks][nb] = half8{0, 0, 0, 0, 0, 0, 0, 0};
+        }
+        multiply(tiles[j]);
+        load_b(t + 1);
+        scatter_slot(std::integral_constant<int, next>{}, tiles[next]);  // tile t + 1 (empty past the end)
+        request(std::integral_constant<int, next>{}, t + 1 + kAhead);
+        clear_quarter(tiles[(j + 2) % 3]);  // tile t - 1, read by all before the last meeting
+        meet();
+    };
+    for (int t = kb; t < ke; t += kAhead) {
+        step(std::integral_constant<int, 0>{}, t);
+        step(std::integral_constant<int, 1>{}, t + 1);
+        step(std::integral_constant<int, 2>{}, t + 2);
+    }
+
+    // the MFMAs came from inline assembly, where the compiler does not pad for the matrix core's write-back
+    // latency: give the last ones time before the accumulators are read
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    // D layout of the 16x16 MFMA: lane holds column r16, rows 4*g .. 4*g+3 of each 16-row block.  The lane's
+    // coordinates are derived afresh (through an opaque statement) so that nothing is carried round the loop for this.
+    int lane_again = threadIdx.x & (kLanes - 1);
+    asm volatile("" : "+v"(lane_again));
+    const int r16 = lane_again & 15, g = lane_again >> 4;
+#pragma unroll
+    for (int nb = 0; nb < NBW; nb++) {
+        const int n = col0 + nb * 16 + r16;
+        if (n < N) {
+#pragma unroll
+            for (int rb = 0; rb < 8; rb++) {
+                half4 h;
+                h[0] = static_cast<_Float16>(acc[nb][rb][0]);
+                h[1] = static_cast<_Float16>(acc[nb][rb][1]);
+                h[2] = static_cast<_Float16>(acc[nb][rb][2]);
+                h[3] = static_cast<_Float16>(acc[nb][rb][3]);
+                *reinterpret_cast<half4*>(o + static_cast<size_t>(n) * M + g * 4 + rb * 16) = h;
+            }
+        }
+    }
+}
+
+template<int NBW>
+__global__ __launch_bounds__(kGroupThreads, 3) void spmm_group_kernel(const uint4* __restrict__ comp,
+                                                                  const int* __restrict__ offs,
+                                                                  const _Float16* __restrict__ B,
+                                                                  _Float16* __restrict__ out,
+                                                                  int M,
+                                                                  int N,
+                                                                  int K,
+                                                                  int split_k,
+                                                                  int col_groups)
+{
+    __shared__ __attribute__((aligned(16))) uint16_t tiles[3][kTileHalfs];
+    const int kt = K / kTileCols;
+    int       unit, slice;
+    unit_of_workgroup(blockIdx.x, gridDim.x / split_k, split_k, unit, slice);
+    const int rowtile = unit / col_groups;
+    const int col0    = (unit % col_groups) * (kGroupWaves * 16 * NBW) + (threadIdx.x / kLanes) * (16 * NBW);
+    // the reference's slicing (csrc/SpMM_Kernel.cuh:196-204), clamped to K
+    const int avg = (kt - 1) / split_k + 1;
+    int       kb  = slice * avg;
+    kb            = kb < kt ? kb : kt;
+    int ke        = kb + avg;
+    ke            = ke < kt ? ke : kt;
+    const int* toff = offs + static_cast<size_t>(rowtile) * kt;
+    _Float16*  o    = out + static_cast<size_t>(slice) * M * N + static_cast<size_t>(rowtile) * kTileRows;
+    // last vector any load of this slice may touch (clamped loads re-read it); vector 0 exists even in an
+    // empty matrix, whose callers allocate at least one
+    int vmax = toff[ke] - 1;
+    vmax     = vmax > 0 ? vmax : 0;
+    // rounds held in registers per tile: two cover 512 vectors (8 KB, tiles up to a quarter full), three 768
+    const int whole = offs[static_cast<size_t>(M / kTileRows) * kt];  // vectors in the matrix
+    if (whole <= 440LL * (M / kTileRows) * kt)
+        spmm_group_body<NBW, 2>(tiles, comp, toff, B, o, M, N, K, kb, ke, col0, vmax);
+    else
+        spmm_group_body<NBW, 3>(tiles, comp, toff, B, o, M, N, K, kb, ke, col0, vmax);
+}
+
 __device__ __forceinline__ void add_slab(float (&s)[4], const uint2 v)
 {
     const half4 h = __builtin_bit_cast(half4, v);
@@ -563,6 +792,17 @@ extern "C" int flashllm_hip_launch_spmm(
     return launch_spmm<4, 6>(s, comp, offs, b, out, m, n, k, split_k, n / 64);
 }
 
+extern "C" int flashllm_hip_launch_spmm_group(
+    void* stream, const void* comp, const int* offs, const void* b, void* out, int m, int n, int k, int split_k)
+{
+    // 128 columns per workgroup (four waves x 32); requires n % 128 == 0
+    const dim3 grid(static_cast<unsigned>(m / kTileRows) * (n / 128) * split_k, 1, 1);
+    hipLaunchKernelGGL(spmm_group_kernel<2>, grid, dim3(kGroupThreads), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint4*>(comp), offs, static_cast<const _Float16*>(b), static_cast<_Float16*>(out),
+                       m, n, k, split_k, n / 128);
+    return static_cast<int>(hipGetLastError());
+}
+
 extern "C" int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws, long mn, int split_k, int relu)
 {
     const long     n4 = mn / 4;
@@ -579,9 +819,11 @@ extern "C" int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws,
 
 extern "C" int flashllm_hip_launch_reduce_blocks(void* stream, void* c, const void* ws, int m, int n, int split_k, int relu)
 {
-    // the units of flashllm_hip_launch_spmm for this N: 16*nb columns wide
-    const int   nb         = n <= 16 ? 1 : (n == 32 ? 2 : 4);
-    const int   col_groups = n <= 64 ? 1 : n / 64;
+    // the units of the SpMM launch for this N, 16*nb columns wide: one wave's columns in spmm_stream_kernel,
+    // a workgroup's 128 in spmm_group_kernel
+    const bool  group      = n % 128 == 0;
+    const int   nb         = group ? 8 : (n <= 16 ? 1 : (n == 32 ? 2 : 4));
+    const int   col_groups = group ? n / 128 : (n <= 64 ? 1 : n / 64);
     const dim3  grid(static_cast<unsigned>(m / kTileRows) * col_groups * nb);
     hipStream_t s  = static_cast<hipStream_t>(stream);
     _Float16*   cp = static_cast<_Float16*>(c);

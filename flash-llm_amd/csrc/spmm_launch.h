@@ -27,6 +27,17 @@ int flashllm_hip_launch_spmm(void*       stream,
                              int         k,
                              int         split_k);
 
+// The same product for wide B (n % 128 == 0) by workgroups of four waves that share each scattered tile.
+int flashllm_hip_launch_spmm_group(void*       stream,
+                                   const void* compressed_a,
+                                   const int*  tile_offsets,
+                                   const void* b,
+                                   void*       out,
+                                   int         m,
+                                   int         n,
+                                   int         k,
+                                   int         split_k);
+
 // c[e] = rn16(sum_s float(ws[s*mn + e])), through max(., 0) first when relu != 0; requires mn % 4 == 0.
 int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws, long mn, int split_k, int relu);
 

@@ -90,6 +90,62 @@ def test_ragged_tiles_and_empty_slices(product, oracle, torch_gpu):
         assert_close(c, ref, f"ragged split_k={split_k}")
 
 
+# --- the four-wave kernel for wide B (N a multiple of 128) -------------------------------------------
+@pytest.mark.parametrize("n", [128, 384])
+@pytest.mark.parametrize("sparsity", [0.0, 0.5, 0.72, 0.8, 0.95, 0.999, 1.0])
+def test_wide_b_any_density(product, oracle, torch_gpu, sparsity, n):
+    """Tiles of up to 512 vectors are held in registers two rounds at a time (three when the matrix is denser
+    than about a quarter); longer ones take further rounds straight from memory.  0 % and 50 % are all long
+    tiles, 72 % mixes both kinds, 99.9 % is mostly empty tiles."""
+    say(f"wide B density sparsity={sparsity} n={n}")
+    a = synth.sparse_matrix(384, 1280, sparsity, 41)
+    b = synth.dense_b(1280, n, 42)
+    for split_k in (1, 3):
+        c, _, _ = run_spmm(product, a, b, n, split_k)
+        _, ref = oracle.spmm_model(a, b, n, split_k)
+        if sparsity == 1.0:
+            assert not c.any()
+        else:
+            assert_close(c, ref, f"wide sparsity={sparsity} n={n} split_k={split_k}")
+
+
+def test_wide_b_ragged_tiles_and_empty_slices(product, oracle, torch_gpu):
+    """The wide kernel always runs whole rounds of three tiles: slices of 1, 2, 3, 4 and 0 tiles, empty tiles at
+    either end, a single-vector tile and a full tile."""
+    say("wide B ragged tiles")
+    m, k, n = 256, 640, 256
+    a = synth.sparse_matrix(m, k, 0.8, 43)
+    a[:128, 0:64] = 0
+    a[:128, 256:384] = 0
+    a[128:, 576:640] = 0
+    a[128:, 64:128] = 0
+    a[130, 70] = 1.5
+    a[:128, 448:512] = synth.sparse_matrix(128, 64, 0.0, 44)
+    b = synth.dense_b(k, n, 45)
+    for split_k in (1, 2, 3, 5, 10, 16):
+        c, _, _ = run_spmm(product, a, b, n, split_k)
+        _, ref = oracle.spmm_model(a, b, n, split_k)
+        assert_close(c, ref, f"wide ragged split_k={split_k}")
+
+
+def test_wide_b_matches_the_narrow_kernel_bit_for_bit(product, torch_gpu):
+    """Both kernels accumulate a slice's k tiles in order with the same MFMA, so their slabs are identical:
+    the 128 columns of a wide call equal two 64-column calls on the column halves."""
+    torch = torch_gpu
+    say("wide B vs narrow kernel")
+    m, k, n, s = 1024, 2048, 128, 4
+    a = synth.sparse_matrix(m, k, 0.8, 46, dist="normal", sigma=0.05)
+    b_h = synth.dense_b(k, n, 47, dist="normal")
+    wide, w, _ = run_spmm(product, a, b_h, n, s)
+    b = torch.from_numpy(b_h).cuda()
+    for half in range(2):
+        c = torch.empty(64 * m, dtype=torch.float16, device="cuda")
+        ws = torch.empty(s * 64 * m, dtype=torch.float16, device="cuda")
+        product.spmm_splitk(w.comp, w.offs, b[half * 64:(half + 1) * 64].contiguous(), c, m, 64, k, ws, s)
+        torch.cuda.synchronize()
+        assert np.array_equal(c.cpu().numpy().view(np.uint16), wide[half * 64:(half + 1) * 64].reshape(-1).view(np.uint16))
+
+
 def test_ones_matrix_subset_sums(product, oracle, torch_gpu):
     """The reference benchmark's data (A in {0,1}, B in fifths): small exact sums."""
     say("ones matrix")

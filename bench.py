@@ -129,7 +129,7 @@ def main():
         F.spmm_splitk(comps[i % len(comps)], offs, b, c, m, n, k, ws, split_k)
 
     def kernel_only(i):
-        F.spmm_partials(comps[i % len(comps)], offs, b, c, m, n, k, ws, split_k)
+        F.spmm_partials(comps[i % len(comps)], offs, b, c, m, n, k, ws, split_k, slab_order=F.SLABS_BY_WORKGROUP)
 
     def settle(fn):
         # The GPU leaves its idle clocks only after a few hundred ms of work (the reference times 10 000

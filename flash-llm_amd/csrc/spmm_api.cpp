@@ -34,12 +34,25 @@ int check_shape(const void* comp, const int* offs, const void* b, const void* c,
     return hipSuccess;
 }
 
-// The reduction behind a SpMM launch of this shape: by blocks of C on the XCD that holds their slabs when the
-// layout allows it (always, for shapes the SpMM kernel takes, unless C is only 8-byte aligned).
-int reduce_slabs(void* stream, void* c, const void* ws, int m, int n, int split_k, int relu)
+bool known_order(int slab_order)
 {
-    if (m % 128 == 0 && supported_n(n) && reinterpret_cast<uintptr_t>(c) % 16 == 0 && reinterpret_cast<uintptr_t>(ws) % 16 == 0)
-        return flashllm_hip_launch_reduce_blocks(stream, c, ws, m, n, split_k, relu);
+    return slab_order == FLASHLLM_SLABS_PLAIN || slab_order == FLASHLLM_SLABS_BY_WORKGROUP;
+}
+
+int launch_partials(void* stream, const void* comp, const int* offs, const void* b, void* c, int m, int n, int k, void* ws, int split_k, int slab_order)
+{
+    const int pages = slab_order == FLASHLLM_SLABS_BY_WORKGROUP;
+    // wide B: four waves share every scattered tile; otherwise one wave per (row tile, slice, column group)
+    if (n % 128 == 0)
+        return flashllm_hip_launch_spmm_group(stream, comp, offs, b, split_k == 1 ? c : ws, m, n, k, split_k, pages);
+    return flashllm_hip_launch_spmm(stream, comp, offs, b, split_k == 1 ? c : ws, m, n, k, split_k, pages);
+}
+
+// The reduction behind launch_partials with the same slab_order.
+int reduce_slabs(void* stream, void* c, const void* ws, int m, int n, int split_k, int relu, int slab_order)
+{
+    if (slab_order == FLASHLLM_SLABS_BY_WORKGROUP)
+        return flashllm_hip_launch_reduce_pages(stream, c, ws, m, n, split_k, relu);
     return flashllm_hip_launch_reduce(stream, c, ws, static_cast<long>(m) * n, split_k, relu);
 }
 
@@ -56,22 +69,26 @@ int flashllm_spmm_partials(void*       stream,
                            int         n,
                            int         k,
                            void*       ws,
-                           int         split_k)
+                           int         split_k,
+                           int         slab_order)
 {
     const int bad = check_shape(comp, offs, b, c, m, n, k, ws, split_k);
     if (bad)
         return bad;
-    // wide B: four waves share every scattered tile; otherwise one wave per (row tile, slice, column group)
-    if (n % 128 == 0)
-        return flashllm_hip_launch_spmm_group(stream, comp, offs, b, split_k == 1 ? c : ws, m, n, k, split_k);
-    return flashllm_hip_launch_spmm(stream, comp, offs, b, split_k == 1 ? c : ws, m, n, k, split_k);
+    if (!known_order(slab_order))
+        return hipErrorInvalidValue;
+    return launch_partials(stream, comp, offs, b, c, m, n, k, ws, split_k, slab_order);
 }
 
-int flashllm_splitk_reduce(void* stream, void* c, const void* ws, int m, int n, int split_k)
+int flashllm_splitk_reduce(void* stream, void* c, const void* ws, int m, int n, int split_k, int slab_order)
 {
-    if (!c || !ws || m <= 0 || n <= 0 || split_k < 1 || (static_cast<long>(m) * n) % 4)
+    if (!c || !ws || m <= 0 || n <= 0 || split_k < 1 || (static_cast<long>(m) * n) % 4 || !known_order(slab_order)
+        || reinterpret_cast<uintptr_t>(c) % 8 || reinterpret_cast<uintptr_t>(ws) % 8)
         return hipErrorInvalidValue;
-    return reduce_slabs(stream, c, ws, m, n, split_k, 0);
+    // pages exist only for shapes the SpMM kernels take
+    if (slab_order == FLASHLLM_SLABS_BY_WORKGROUP && (m % 128 || !supported_n(n) || reinterpret_cast<uintptr_t>(ws) % 16))
+        return hipErrorInvalidValue;
+    return reduce_slabs(stream, c, ws, m, n, split_k, 0, slab_order);
 }
 
 int flashllm_spmm_splitk(void*       stream,
@@ -86,10 +103,11 @@ int flashllm_spmm_splitk(void*       stream,
                          void*       ws,
                          int         split_k)
 {
-    int rc = flashllm_spmm_partials(stream, comp, offs, b, c, m, n, k, ws, split_k);
+    // the workspace is this call's own business between its two kernels: slabs by workgroup
+    int rc = flashllm_spmm_partials(stream, comp, offs, b, c, m, n, k, ws, split_k, FLASHLLM_SLABS_BY_WORKGROUP);
     if (rc || split_k == 1)
         return rc;
-    return reduce_slabs(stream, c, ws, m, n, split_k, 0);
+    return reduce_slabs(stream, c, ws, m, n, split_k, 0, FLASHLLM_SLABS_BY_WORKGROUP);
 }
 
 // SpMM_SplitK_API for callers that must not allocate and hold no workspace: the slabs go to the
@@ -261,10 +279,10 @@ int flashllm_decoder_layer_linears(void*                         stream,
         return rc;
     // FFN1 with the ReLU folded into its reduction when there is one
     const int s1 = split(f1, 128);
-    rc = flashllm_spmm_partials(stream, f1.nz_weights, f1.tile_offsets, attn_out, ffn_mid, f1.m, tokens, f1.k, ws, s1);
+    rc = flashllm_spmm_partials(stream, f1.nz_weights, f1.tile_offsets, attn_out, ffn_mid, f1.m, tokens, f1.k, ws, s1, FLASHLLM_SLABS_BY_WORKGROUP);
     if (rc)
         return rc;
-    rc = s1 > 1 ? reduce_slabs(stream, ffn_mid, ws, f1.m, tokens, s1, 1)
+    rc = s1 > 1 ? reduce_slabs(stream, ffn_mid, ws, f1.m, tokens, s1, 1, FLASHLLM_SLABS_BY_WORKGROUP)
                 : flashllm_hip_launch_relu(stream, ffn_mid, static_cast<long>(f1.m) * tokens);
     if (rc)
         return rc;

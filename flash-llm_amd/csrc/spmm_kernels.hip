@@ -37,15 +37,15 @@
 //
 // Placement.  The GPU has eight accelerator dies (XCDs), each with its own L2, and hands the
 // workgroups of a launch to them round-robin in launch order: workgroup w runs on XCD w % 8.  The
-// SpMM kernel therefore gives the Split_K slices of one (row tile, column group) unit to workgroups
-// eight apart, and each XCD a contiguous block of units: the slabs of a unit all land in one L2.
+// SpMM kernels therefore give the Split_K slices of one (row tile, column group) unit to workgroups
+// eight apart, and each XCD a contiguous block of units: the partial sums of a unit all land in one L2.
 //
-// splitk_reduce_block_kernel: the separate reduction over fp16 slabs (reference
-// csrc/Reduction_Kernel.cuh:24-45), one workgroup per 128 x 16 block of C, given to the XCD whose L2
-// holds that block's slabs (the lines survive the kernel boundary), 16 bytes per lane per slab, eight
-// slabs in flight.  Where a workgroup runs only decides where its loads hit; the sums do not depend on it.
-// splitk_reduce_kernel: the same sums over a flat M*N range, for outputs the block kernel's layout does
-// not cover.
+// splitk_reduce_pages_kernel: the separate reduction (reference csrc/Reduction_Kernel.cuh:24-45) over
+// slabs stored by workgroup (store_pages below), one workgroup per 128 x 16 block of C on the XCD that
+// stored the block's pages, 16 bytes per lane per slice, eight slices in flight.  Where a workgroup runs
+// only decides where its loads hit; the sums do not depend on it.
+// splitk_reduce_kernel: the same sums over plain slabs (slab s = M*N halfs laid out like C), the
+// reference's workspace layout.
 #include "spmm_launch.h"
 
 #include <hip/hip_runtime.h>
@@ -82,6 +82,46 @@ __device__ __forceinline__ void unit_of_workgroup(unsigned w, unsigned units, un
     else {
         unit = static_cast<int>(w / parts);
         part = static_cast<int>(w % parts);
+    }
+}
+
+// The inverse: which workgroup of the launch has (unit, part).
+__device__ __forceinline__ unsigned workgroup_of_unit(unsigned unit, unsigned part, unsigned units, unsigned parts)
+{
+    const unsigned per_xcd = units / kXcds;
+    if (unit < per_xcd * kXcds)
+        return ((unit % per_xcd) * parts + part) * kXcds + unit / per_xcd;
+    return unit * parts + part;
+}
+
+// Slab storage by workgroup ("pages").  A page is one 128-row x 16-column block of partial sums (4 KB; 128 x 8
+// and 2 KB when N == 8), kept in the order the matrix cores leave it in registers: 16-byte piece
+// q*(4*cols) + g*cols + r16 holds rows 32q + 4g .. +3 and 32q + 16 + 4g .. +3 of column r16.  Page b of
+// workgroup w of a launch of G workgroups is page b*G + w of the workspace.  Under round-robin hand-out the
+// XCD that writes and later sums a page is (page index) % 8 whenever G is a multiple of 8, whatever the shape
+// of the product: a workspace shared by the linears of a layer keeps every line in one L2, where stores to
+// lines already present stay readable for the reduction kernel (stores that miss go to memory and do not).
+template<int NBLK>
+__device__ __forceinline__ void store_pages(_Float16* ws, const floatx4 (&acc)[NBLK][8], int first_page, int N, int lane)
+{
+    const int    cols  = N < 16 ? 8 : 16;
+    const int    r16   = lane & 15, g = lane >> 4;
+    const size_t pitch = static_cast<size_t>(gridDim.x) * (cols * 16);  // uint4 between consecutive pages of a workgroup
+    uint4*       page  = reinterpret_cast<uint4*>(ws) + (static_cast<size_t>(first_page) * gridDim.x + blockIdx.x) * (cols * 16);
+    if (r16 >= cols)
+        return;
+#pragma unroll
+    for (int nb = 0; nb < NBLK; nb++) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            half8 h;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                h[e]     = static_cast<_Float16>(acc[nb][2 * q][e]);
+                h[4 + e] = static_cast<_Float16>(acc[nb][2 * q + 1][e]);
+            }
+            page[nb * pitch + q * (4 * cols) + g * cols + r16] = __builtin_bit_cast(uint4, h);
+        }
     }
 }
 
@@ -191,7 +231,8 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                                                             int N,
                                                             int K,
                                                             int split_k,
-                                                            int col_groups)
+                                                            int col_groups,
+                                                            int pages)
 {
     __shared__ __attribute__((aligned(16))) uint16_t tile[kTileHalfs];
 
@@ -349,6 +390,10 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
     }
 
     // D layout of the 16x16 MFMA: lane holds column r16, rows 4*g .. 4*g+3 of each 16-row block.
+    if (pages) {
+        store_pages<NB>(out, acc, 0, N, lane);
+        return;
+    }
     _Float16* o = out + static_cast<size_t>(slice) * M * N + static_cast<size_t>(rowtile) * kTileRows + g * 4;
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) {
@@ -400,7 +445,8 @@ __device__ __forceinline__ void spmm_group_body(uint16_t (&tiles)[3][kTileHalfs]
                                                 int kb,
                                                 int ke,
                                                 int col0,
-                                                int vmax)
+                                                int vmax,
+                                                int pages)
 {
     const int lane = threadIdx.x & (kLanes - 1);
     const int wave = threadIdx.x / kLanes;
@@ -540,6 +586,10 @@ __device__ __forceinline__ void spmm_group_body(uint16_t (&tiles)[3][kTileHalfs]
     // coordinates are derived afresh (through an opaque statement) so that nothing is carried round the loop for this.
     int lane_again = threadIdx.x & (kLanes - 1);
     asm volatile("" : "+v"(lane_again));
+    if (pages) {  // o is the workspace itself here; this wave's NBW pages follow those of the waves before it
+        store_pages<NBW>(o, acc, static_cast<int>(threadIdx.x / kLanes) * NBW, N, lane_again);
+        return;
+    }
     const int r16 = lane_again & 15, g = lane_again >> 4;
 #pragma unroll
     for (int nb = 0; nb < NBW; nb++) {
@@ -567,7 +617,8 @@ __global__ __launch_bounds__(kGroupThreads, 3) void spmm_group_kernel(const uint
                                                                   int N,
                                                                   int K,
                                                                   int split_k,
-                                                                  int col_groups)
+                                                                  int col_groups,
+                                                                  int pages)
 {
     __shared__ __attribute__((aligned(16))) uint16_t tiles[3][kTileHalfs];
     const int kt = K / kTileCols;
@@ -582,7 +633,7 @@ __global__ __launch_bounds__(kGroupThreads, 3) void spmm_group_kernel(const uint
     int ke        = kb + avg;
     ke            = ke < kt ? ke : kt;
     const int* toff = offs + static_cast<size_t>(rowtile) * kt;
-    _Float16*  o    = out + static_cast<size_t>(slice) * M * N + static_cast<size_t>(rowtile) * kTileRows;
+    _Float16*  o    = pages ? out : out + static_cast<size_t>(slice) * M * N + static_cast<size_t>(rowtile) * kTileRows;
     // last vector any load of this slice may touch (clamped loads re-read it); vector 0 exists even in an
     // empty matrix, whose callers allocate at least one
     int vmax = toff[ke] - 1;
@@ -590,9 +641,9 @@ __global__ __launch_bounds__(kGroupThreads, 3) void spmm_group_kernel(const uint
     // rounds held in registers per tile: two cover 512 vectors (8 KB, tiles up to a quarter full), three 768
     const int whole = offs[static_cast<size_t>(M / kTileRows) * kt];  // vectors in the matrix
     if (whole <= 440LL * (M / kTileRows) * kt)
-        spmm_group_body<NBW, 2>(tiles, comp, toff, B, o, M, N, K, kb, ke, col0, vmax);
+        spmm_group_body<NBW, 2>(tiles, comp, toff, B, o, M, N, K, kb, ke, col0, vmax, pages);
     else
-        spmm_group_body<NBW, 3>(tiles, comp, toff, B, o, M, N, K, kb, ke, col0, vmax);
+        spmm_group_body<NBW, 3>(tiles, comp, toff, B, o, M, N, K, kb, ke, col0, vmax, pages);
 }
 
 __device__ __forceinline__ void add_slab(float (&s)[4], const uint2 v)
@@ -656,34 +707,35 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(uint2* __restrict__ 
     c[i] = __builtin_bit_cast(uint2, h);
 }
 
-// The same sums for the output of spmm_stream_kernel, one workgroup per 128-row x 16-column block of C:
-// lane = (column, 16-byte piece of the column's 128 rows).  blocks_per_unit: 16-column blocks of one unit
-// of the SpMM kernel (its NB); the workgroup order mirrors that kernel's, so a block is summed on the XCD
-// that stored its slabs.
+// The same sums over slabs stored by workgroup (store_pages), one workgroup per 128-row x 16-column block of C.
+// pages_per_unit: pages one workgroup of the SpMM launch stores (its NB, or 4*NBW in the four-wave kernel);
+// spmm_grid: workgroups of that launch.  The workgroup order mirrors the SpMM kernel's, so a block is summed
+// on the XCD that stored its pages.  Thread t takes 16-byte piece t of each slice's page.
 template<bool RELU>
-__global__ __launch_bounds__(256) void splitk_reduce_block_kernel(_Float16* __restrict__ c,
-                                                                 const _Float16* __restrict__ ws,
+__global__ __launch_bounds__(256) void splitk_reduce_pages_kernel(_Float16* __restrict__ c,
+                                                                 const uint4* __restrict__ ws,
                                                                  int M,
                                                                  int N,
                                                                  int split_k,
-                                                                 int blocks_per_unit,
-                                                                 int col_groups)
+                                                                 int pages_per_unit,
+                                                                 int col_groups,
+                                                                 unsigned spmm_grid)
 {
-    int unit, sub;
-    unit_of_workgroup(blockIdx.x, gridDim.x / blocks_per_unit, blocks_per_unit, unit, sub);
-    const int rowtile = unit / col_groups;
-    const int n       = ((unit % col_groups) * blocks_per_unit + sub) * 16 + (threadIdx.x >> 4);
-    if (n >= N)  // N == 8: half a block
+    const int cols = N < 16 ? 8 : 16;
+    const int t    = threadIdx.x;
+    if (t >= cols * 16)  // N == 8: half a block
         return;
-    const size_t slab = static_cast<size_t>(M) * N;
-    const size_t at   = static_cast<size_t>(n) * M + static_cast<size_t>(rowtile) * kTileRows + (threadIdx.x & 15) * 8;
-    float        s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const unsigned units = gridDim.x / pages_per_unit;
+    int            unit, sub;
+    unit_of_workgroup(blockIdx.x, units, pages_per_unit, unit, sub);
+    const uint4* first = ws + static_cast<size_t>(sub) * spmm_grid * (cols * 16) + t;
+    float        s[8]  = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int k0 = 0; k0 < split_k; k0 += 8) {
         uint4 v[8];
 #pragma unroll
         for (int j = 0; j < 8; j++)
             if (k0 + j < split_k)
-                v[j] = *reinterpret_cast<const uint4*>(ws + (k0 + j) * slab + at);
+                v[j] = first[static_cast<size_t>(workgroup_of_unit(unit, k0 + j, units, split_k)) * (cols * 16)];
 #pragma unroll
         for (int j = 0; j < 8; j++)
             if (k0 + j < split_k) {
@@ -693,11 +745,18 @@ __global__ __launch_bounds__(256) void splitk_reduce_block_kernel(_Float16* __re
                     s[e] += static_cast<float>(h[e]);
             }
     }
-    half8 h;
+    half4 lo, hi;
 #pragma unroll
-    for (int e = 0; e < 8; e++)
-        h[e] = static_cast<_Float16>(RELU && !(s[e] > 0.f) ? 0.f : s[e]);
-    *reinterpret_cast<uint4*>(c + at) = __builtin_bit_cast(uint4, h);
+    for (int e = 0; e < 4; e++) {
+        lo[e] = static_cast<_Float16>(RELU && !(s[e] > 0.f) ? 0.f : s[e]);
+        hi[e] = static_cast<_Float16>(RELU && !(s[4 + e] > 0.f) ? 0.f : s[4 + e]);
+    }
+    // piece t = q*(4*cols) + g*cols + r16: rows 32q + 4g .. +3 and 16 further on, column r16 of the block
+    const int q = t / (4 * cols), g = (t / cols) & 3, r16 = t % cols;
+    const int n = ((unit % col_groups) * pages_per_unit + sub) * 16 + r16;
+    _Float16* o = c + static_cast<size_t>(n) * M + static_cast<size_t>(unit / col_groups) * kTileRows + q * 32 + g * 4;
+    *reinterpret_cast<half4*>(o)      = lo;
+    *reinterpret_cast<half4*>(o + 16) = hi;
 }
 
 // out[w] = id of the XCD that workgroup w of this launch ran on
@@ -729,7 +788,7 @@ __global__ __launch_bounds__(256) void take_rows_kernel(uint4* __restrict__ dst,
 }
 
 template<int NB, int DEPTH>
-int launch_spmm(hipStream_t stream, const void* comp, const int* offs, const void* b, void* out, int m, int n, int k, int split_k, int col_groups)
+int launch_spmm(hipStream_t stream, const void* comp, const int* offs, const void* b, void* out, int m, int n, int k, int split_k, int col_groups, int pages)
 {
     const dim3 grid(static_cast<unsigned>(m / kTileRows) * col_groups * split_k, 1, 1);
     hipLaunchKernelGGL((spmm_stream_kernel<NB, DEPTH>),
@@ -745,7 +804,8 @@ int launch_spmm(hipStream_t stream, const void* comp, const int* offs, const voi
                        n,
                        k,
                        split_k,
-                       col_groups);
+                       col_groups,
+                       pages);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -781,25 +841,27 @@ extern "C" int flashllm_hip_static_workspace(void** ptr)
     return 0;
 }
 
+// pages != 0 (Split_K > 1 only): the slabs go to the workspace by workgroup, for flashllm_hip_launch_reduce_pages
 extern "C" int flashllm_hip_launch_spmm(
-    void* stream, const void* comp, const int* offs, const void* b, void* out, int m, int n, int k, int split_k)
+    void* stream, const void* comp, const int* offs, const void* b, void* out, int m, int n, int k, int split_k, int pages)
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
+    pages         = pages && split_k > 1;
     if (n <= 16)
-        return launch_spmm<1, 8>(s, comp, offs, b, out, m, n, k, split_k, 1);
+        return launch_spmm<1, 8>(s, comp, offs, b, out, m, n, k, split_k, 1, pages);
     if (n == 32)
-        return launch_spmm<2, 8>(s, comp, offs, b, out, m, n, k, split_k, 1);
-    return launch_spmm<4, 6>(s, comp, offs, b, out, m, n, k, split_k, n / 64);
+        return launch_spmm<2, 8>(s, comp, offs, b, out, m, n, k, split_k, 1, pages);
+    return launch_spmm<4, 6>(s, comp, offs, b, out, m, n, k, split_k, n / 64, pages);
 }
 
 extern "C" int flashllm_hip_launch_spmm_group(
-    void* stream, const void* comp, const int* offs, const void* b, void* out, int m, int n, int k, int split_k)
+    void* stream, const void* comp, const int* offs, const void* b, void* out, int m, int n, int k, int split_k, int pages)
 {
     // 128 columns per workgroup (four waves x 32); requires n % 128 == 0
     const dim3 grid(static_cast<unsigned>(m / kTileRows) * (n / 128) * split_k, 1, 1);
     hipLaunchKernelGGL(spmm_group_kernel<2>, grid, dim3(kGroupThreads), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint4*>(comp), offs, static_cast<const _Float16*>(b), static_cast<_Float16*>(out),
-                       m, n, k, split_k, n / 128);
+                       m, n, k, split_k, n / 128, pages && split_k > 1);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -817,21 +879,22 @@ extern "C" int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws,
     return static_cast<int>(hipGetLastError());
 }
 
-extern "C" int flashllm_hip_launch_reduce_blocks(void* stream, void* c, const void* ws, int m, int n, int split_k, int relu)
+extern "C" int flashllm_hip_launch_reduce_pages(void* stream, void* c, const void* ws, int m, int n, int split_k, int relu)
 {
     // the units of the SpMM launch for this N, 16*nb columns wide: one wave's columns in spmm_stream_kernel,
     // a workgroup's 128 in spmm_group_kernel
-    const bool  group      = n % 128 == 0;
-    const int   nb         = group ? 8 : (n <= 16 ? 1 : (n == 32 ? 2 : 4));
-    const int   col_groups = group ? n / 128 : (n <= 64 ? 1 : n / 64);
-    const dim3  grid(static_cast<unsigned>(m / kTileRows) * col_groups * nb);
-    hipStream_t s  = static_cast<hipStream_t>(stream);
-    _Float16*   cp = static_cast<_Float16*>(c);
-    const _Float16* wp = static_cast<const _Float16*>(ws);
+    const bool     group      = n % 128 == 0;
+    const int      nb         = group ? 8 : (n <= 16 ? 1 : (n == 32 ? 2 : 4));
+    const int      col_groups = group ? n / 128 : (n <= 64 ? 1 : n / 64);
+    const unsigned units      = static_cast<unsigned>(m / kTileRows) * col_groups;
+    const dim3     grid(units * nb);
+    hipStream_t    s  = static_cast<hipStream_t>(stream);
+    _Float16*      cp = static_cast<_Float16*>(c);
+    const uint4*   wp = static_cast<const uint4*>(ws);
     if (relu)
-        hipLaunchKernelGGL(splitk_reduce_block_kernel<true>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, nb, col_groups);
+        hipLaunchKernelGGL(splitk_reduce_pages_kernel<true>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, nb, col_groups, units * split_k);
     else
-        hipLaunchKernelGGL(splitk_reduce_block_kernel<false>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, nb, col_groups);
+        hipLaunchKernelGGL(splitk_reduce_pages_kernel<false>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, nb, col_groups, units * split_k);
     return static_cast<int>(hipGetLastError());
 }
 

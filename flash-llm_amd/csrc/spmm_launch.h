@@ -16,6 +16,9 @@ extern "C" {
 int flashllm_hip_static_workspace(void** ptr);
 
 // out: C when split_k == 1, else the slab workspace (split_k * M * N halfs).
+// pages == 0: slab s is M*N halfs at s*M*N, laid out like C (for flashllm_hip_launch_reduce);
+// pages != 0: each workgroup's 128 x 16 blocks of partial sums as 4 KB pages in workgroup order
+// (for flashllm_hip_launch_reduce_pages; needs out 16-byte aligned).
 // Requires M % 128 == 0, K % 64 == 0, N in {8,16,32,64} or N % 64 == 0.
 int flashllm_hip_launch_spmm(void*       stream,
                              const void* compressed_a,
@@ -25,7 +28,8 @@ int flashllm_hip_launch_spmm(void*       stream,
                              int         m,
                              int         n,
                              int         k,
-                             int         split_k);
+                             int         split_k,
+                             int         pages);
 
 // The same product for wide B (n % 128 == 0) by workgroups of four waves that share each scattered tile.
 int flashllm_hip_launch_spmm_group(void*       stream,
@@ -36,14 +40,16 @@ int flashllm_hip_launch_spmm_group(void*       stream,
                                    int         m,
                                    int         n,
                                    int         k,
-                                   int         split_k);
+                                   int         split_k,
+                                   int         pages);
 
 // c[e] = rn16(sum_s float(ws[s*mn + e])), through max(., 0) first when relu != 0; requires mn % 4 == 0.
 int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws, long mn, int split_k, int relu);
 
-// The same sums for the slabs flashllm_hip_launch_spmm left for this (m, n): one workgroup per 128 x 16 block
-// of C, on the XCD whose L2 holds the block's slabs.  Requires M % 128 == 0, N as above, c and ws 16-byte aligned.
-int flashllm_hip_launch_reduce_blocks(void* stream, void* c, const void* ws, int m, int n, int split_k, int relu);
+// The same sums over the pages a launch with pages != 0 left for this (m, n, split_k): one workgroup per
+// 128 x 16 block of C, on the XCD that stored the block's pages.  Requires M % 128 == 0, N as above, ws 16-byte
+// and c 8-byte aligned.
+int flashllm_hip_launch_reduce_pages(void* stream, void* c, const void* ws, int m, int n, int split_k, int relu);
 
 // out[w] = id of the XCD workgroup w ran on, for a launch of `workgroups` one-wave workgroups: shows whether
 // the round-robin hand-out the placement above counts on holds on this machine.

@@ -43,8 +43,8 @@ SIGNATURES = {
     "flashllm_set_compress_threads": (None, [ctypes.c_int]),
     "flashllm_spmm_splitk": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int]),
     "flashllm_spmm_splitk_static": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
-    "flashllm_spmm_partials": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int]),
-    "flashllm_splitk_reduce": (ctypes.c_int, [_vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "flashllm_spmm_partials": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int, ctypes.c_int]),
+    "flashllm_splitk_reduce": (ctypes.c_int, [_vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "flashllm_device_tile_offsets": (ctypes.c_int, [_vp, _vp, ctypes.c_int, ctypes.c_int, _vp, ctypes.POINTER(ctypes.c_longlong)]),
     "flashllm_device_compress": (ctypes.c_int, [_vp, _vp, ctypes.c_int, ctypes.c_int, _vp, _vp]),
     "flashllm_splitk_heuristic": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
@@ -183,14 +183,19 @@ def spmm_splitk_static(comp, offs, b, c, m, n, k, split_k, stream=None):
         raise HipError(rc)
 
 
-def spmm_partials(comp, offs, b, c, m, n, k, workspace, split_k, stream=None):
-    rc = lib().flashllm_spmm_partials(_stream(stream), _ptr(comp), _ptr(offs), _ptr(b), _ptr(c), m, n, k, _ptr(workspace), split_k)
+SLABS_PLAIN = 0          # FLASHLLM_SLABS_PLAIN: slab s = M*N halfs at s*M*N, laid out like C
+SLABS_BY_WORKGROUP = 1   # FLASHLLM_SLABS_BY_WORKGROUP: what spmm_splitk keeps between its two kernels
+
+
+def spmm_partials(comp, offs, b, c, m, n, k, workspace, split_k, stream=None, slab_order=SLABS_PLAIN):
+    rc = lib().flashllm_spmm_partials(_stream(stream), _ptr(comp), _ptr(offs), _ptr(b), _ptr(c), m, n, k, _ptr(workspace), split_k,
+                                      slab_order)
     if rc:
         raise HipError(rc)
 
 
-def splitk_reduce(c, workspace, m, n, split_k, stream=None):
-    rc = lib().flashllm_splitk_reduce(_stream(stream), _ptr(c), _ptr(workspace), m, n, split_k)
+def splitk_reduce(c, workspace, m, n, split_k, stream=None, slab_order=SLABS_PLAIN):
+    rc = lib().flashllm_splitk_reduce(_stream(stream), _ptr(c), _ptr(workspace), m, n, split_k, slab_order)
     if rc:
         raise HipError(rc)
 

@@ -59,7 +59,7 @@ def run_case(torch, name, a, n, split_k=None, b_dist="normal", dense=True, copie
     c = torch.empty(n * m, dtype=torch.float16, device="cuda")
     ws = torch.empty(max(1, s) * n * m, dtype=torch.float16, device="cuda")
     ms = timed(torch, lambda i: F.spmm_splitk(comps[i % copies], offs, b, c, m, n, k, ws, s))
-    ms_kernel = timed(torch, lambda i: F.spmm_partials(comps[i % copies], offs, b, c, m, n, k, ws, s))
+    ms_kernel = timed(torch, lambda i: F.spmm_partials(comps[i % copies], offs, b, c, m, n, k, ws, s, slab_order=F.SLABS_BY_WORKGROUP))
     F.spmm_splitk(comps[0], offs, b, c, m, n, k, ws, s)
     torch.cuda.synchronize()
     rows = np.arange(0, m, max(1, m // 256))

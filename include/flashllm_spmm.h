@@ -83,10 +83,29 @@ int flashllm_spmm_splitk_static(void*       stream,
                                 int         Split_K);
 
 /*
+ * Where the two halves below keep the Split_K partial products in
+ * Reduction_Workspace (Split_K*M*N halfs either way):
+ *  FLASHLLM_SLABS_PLAIN         slab s is M*N halfs at s*M*N, laid out like C:
+ *                               the reference's workspace
+ *                               (csrc/SpMM_Kernel.cuh:188-190, :293-303);
+ *  FLASHLLM_SLABS_BY_WORKGROUP  the 128x16 blocks of partial sums as 4 KB
+ *                               pages in the order of the SpMM launch's
+ *                               workgroups, which keeps every page in the L2
+ *                               of the one XCD that writes and sums it.  This
+ *                               is what flashllm_spmm_splitk does between its
+ *                               own two kernels; the contents mean something
+ *                               only to flashllm_splitk_reduce with the same
+ *                               M, N, Split_K.
+ */
+#define FLASHLLM_SLABS_PLAIN 0
+#define FLASHLLM_SLABS_BY_WORKGROUP 1
+
+/*
  * The first half of flashllm_spmm_splitk alone (reference
  * csrc/SpMM_API.cu:73-118): launches only the SpMM kernel and leaves the
- * Split_K fp16 slabs in Reduction_Workspace (or writes C when Split_K == 1).
- * For callers that time the kernels separately or fuse the reduction.
+ * Split_K fp16 slabs in Reduction_Workspace in the given order (or writes C
+ * when Split_K == 1).  For callers that time the kernels separately or fuse
+ * the reduction.
  */
 int flashllm_spmm_partials(void*       stream,
                            const void* Compressed_A,
@@ -97,11 +116,13 @@ int flashllm_spmm_partials(void*       stream,
                            int         N,
                            int         K,
                            void*       Reduction_Workspace,
-                           int         Split_K);
+                           int         Split_K,
+                           int         Slab_Order);
 
 /* The second half alone (reference csrc/Reduction_Kernel.cuh:24-45, launch
- * csrc/SpMM_API.cu:126-128): C[e] = rn16(sum_s float(ws[s*M*N + e])). */
-int flashllm_splitk_reduce(void* stream, void* C, const void* Reduction_Workspace, int M, int N, int Split_K);
+ * csrc/SpMM_API.cu:126-128): C[e] = rn16(sum_s float(slab s at e)), slabs
+ * taken in order, for slabs stored in Slab_Order. */
+int flashllm_splitk_reduce(void* stream, void* C, const void* Reduction_Workspace, int M, int N, int Split_K, int Slab_Order);
 
 /*
  * Split_K recommended for one MI355X (256 CUs, wave64).  Takes the place of

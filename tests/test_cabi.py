@@ -51,7 +51,9 @@ def test_spmm_rejects_bad_arguments_before_any_launch(product):
     assert call(comp=ok + 4) == INVALID
     assert call(n=24) == UNKNOWN       # the reference prints and returns cudaErrorUnknown for such N
     assert call(n=192) == UNKNOWN
-    assert L.flashllm_splitk_reduce(None, None, ok, 128, 8, 2) == INVALID
+    assert L.flashllm_splitk_reduce(None, None, ok, 128, 8, 2, 0) == INVALID
+    assert L.flashllm_splitk_reduce(None, ok, ok, 128, 8, 2, 2) == INVALID   # no such slab order
+    assert L.flashllm_splitk_reduce(None, ok, ok, 100, 8, 2, 1) == INVALID   # pages exist only for M % 128 == 0
 
 
 def test_workspace_and_heuristic(product):

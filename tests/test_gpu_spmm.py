@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 
 import synth
-from gpu_util import assert_close, errors, run_spmm
+from gpu_util import assert_close, errors, run_spmm, slab_pages, slabs_from_pages
 
 pytestmark = pytest.mark.gpu
 
@@ -191,13 +191,31 @@ def test_split_k_reduction_bit_exact(product, oracle, torch_gpu):
     torch = torch_gpu
     say("reduction kernel")
     rng = np.random.default_rng(2)
-    # the last two shapes are outside the SpMM kernel's (M % 128, N) grid: the flat kernel sums those
+    # plain slabs; the last two shapes are outside the SpMM kernel's (M % 128, N) grid
     for m, n, s in [(128, 8, 2), (1024, 16, 7), (256, 64, 32), (384, 8, 5), (2048, 32, 9), (1024, 128, 3), (256, 256, 11),
                     (100, 8, 3), (128, 20, 6)]:
         ws_h = (rng.standard_normal((s, n * m)) * 3).astype(np.float16)
         ws = torch.from_numpy(ws_h).cuda()
         c = torch.zeros(n * m, dtype=torch.float16, device="cuda")
         product.splitk_reduce(c, ws, m, n, s)
+        torch.cuda.synchronize()
+        want = oracle.splitk_reduce(ws_h, n * m, s)
+        assert np.array_equal(c.cpu().numpy().view(np.uint16), want.view(np.uint16))
+
+
+def test_split_k_reduction_of_slabs_by_workgroup_bit_exact(product, oracle, torch_gpu):
+    """The same sums when the slabs lie in the order the library's own two kernels use: random slabs are put
+    into that order on the host (from the layout's description) and must reduce to the oracle's C."""
+    torch = torch_gpu
+    rng = np.random.default_rng(21)
+    # 8 and 16 row tiles fill whole XCD rounds, 1 / 3 / 11 leave units beyond a multiple of eight
+    for m, n, s in [(128, 8, 2), (1024, 16, 7), (256, 64, 32), (384, 8, 5), (2048, 32, 9), (1024, 128, 3), (256, 256, 11),
+                    (1408, 16, 4), (1408, 64, 3)]:
+        say(f"reduction of pages m={m} n={n} s={s}")
+        ws_h = (rng.standard_normal((s, n * m)) * 3).astype(np.float16)
+        ws = torch.from_numpy(slab_pages(ws_h, m, n)).cuda()
+        c = torch.full((n * m,), float("nan"), dtype=torch.float16, device="cuda")
+        product.splitk_reduce(c, ws, m, n, s, slab_order=product.SLABS_BY_WORKGROUP)
         torch.cuda.synchronize()
         want = oracle.splitk_reduce(ws_h, n * m, s)
         assert np.array_equal(c.cpu().numpy().view(np.uint16), want.view(np.uint16))
@@ -215,20 +233,23 @@ def test_workgroups_go_round_robin_over_the_xcds(product, torch_gpu):
     assert distinct in (1, 2, 4, 8)  # whole GPU, or one of its partition modes
 
 
-def test_partials_then_reduce_equals_api(product, oracle, torch_gpu):
+@pytest.mark.parametrize("m,n,k,s", [(512, 16, 1024, 4), (1152, 8, 512, 3), (1280, 64, 512, 2), (384, 128, 768, 3)])
+def test_partials_then_reduce_equals_api(product, oracle, torch_gpu, m, n, k, s):
+    """Both slab orders hold the same partial sums (each the oracle's product over its K slice), and the
+    two halves called separately give the API's C in either order."""
     torch = torch_gpu
-    say("partials + reduce")
-    m, n, k, s = 512, 16, 1024, 4
+    say(f"partials + reduce m={m} n={n} k={k} s={s}")
     a = synth.sparse_matrix(m, k, 0.8, 13)
     b_h = synth.dense_b(k, n, 14)
     c_api, w, ws_api = run_spmm(product, a, b_h, n, s)
     b = torch.from_numpy(b_h).cuda()
-    ws = torch.zeros(s * n * m, dtype=torch.float16, device="cuda")
+    ws = torch.full((s * n * m,), float("nan"), dtype=torch.float16, device="cuda")
     c = torch.zeros(n * m, dtype=torch.float16, device="cuda")
     product.spmm_partials(w.comp, w.offs, b, c, m, n, k, ws, s)
     torch.cuda.synchronize()
     slabs = ws.cpu().numpy().reshape(s, n, m)
-    assert np.array_equal(slabs.view(np.uint16), ws_api.cpu().numpy().reshape(s, n, m).view(np.uint16))
+    # the API call left the same numbers, by workgroup
+    assert np.array_equal(slabs.view(np.uint16), slabs_from_pages(ws_api.cpu().numpy(), s, m, n).view(np.uint16))
     for i, (kb, ke) in enumerate(oracle.splitk_ranges(k, s)):
         _, ref = oracle.spmm_model(np.ascontiguousarray(a[:, kb * 64:ke * 64]), np.ascontiguousarray(b_h[:, kb * 64:ke * 64]), n, 1)
         assert_close(slabs[i], ref, f"slab {i}")
@@ -236,6 +257,14 @@ def test_partials_then_reduce_equals_api(product, oracle, torch_gpu):
     torch.cuda.synchronize()
     assert np.array_equal(c.cpu().numpy().view(np.uint16), c_api.reshape(-1).view(np.uint16))
     assert np.array_equal(c_api.reshape(-1).view(np.uint16), oracle.splitk_reduce(slabs.reshape(s, -1), n * m, s).view(np.uint16))
+    # and the two halves in the library's own order
+    ws2 = torch.full((s * n * m,), float("nan"), dtype=torch.float16, device="cuda")
+    c2 = torch.full((n * m,), float("nan"), dtype=torch.float16, device="cuda")
+    product.spmm_partials(w.comp, w.offs, b, c2, m, n, k, ws2, s, slab_order=product.SLABS_BY_WORKGROUP)
+    product.splitk_reduce(c2, ws2, m, n, s, slab_order=product.SLABS_BY_WORKGROUP)
+    torch.cuda.synchronize()
+    assert np.array_equal(ws2.cpu().numpy().view(np.uint16), ws_api.cpu().numpy().view(np.uint16))
+    assert np.array_equal(c2.cpu().numpy().view(np.uint16), c_api.reshape(-1).view(np.uint16))
 
 
 def test_runs_on_a_side_stream_and_is_repeatable(product, oracle, torch_gpu):

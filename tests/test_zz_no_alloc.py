@@ -25,10 +25,11 @@ def one_call(product, torch, oracle, m, k, n, split_k, seed):
     product.spmm_splitk(w.comp, w.offs, b, want, m, n, k, ws, split_k)
     got = torch.full((n * m,), float("nan"), dtype=torch.float16, device="cuda")
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # cumulative count of allocations made through torch (frees by the garbage collector do not touch it)
+    before = torch.cuda.memory_stats()["allocation.all.allocated"]
     product.spmm_splitk_static(w.comp, w.offs, b, got, m, n, k, split_k)
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
     got_h, want_h = got.cpu().numpy(), want.cpu().numpy()
     assert np.array_equal(got_h.view(np.uint16), want_h.view(np.uint16))
     ref, _ = oracle.gemm_f32(a, b_h, n)

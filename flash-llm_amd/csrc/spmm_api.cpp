@@ -5,6 +5,7 @@
 #include "flashllm_spmm.h"
 #include "spmm_launch.h"
 
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 
@@ -199,18 +200,19 @@ int flashllm_splitk_heuristic(int m, int n, int k)
     if (n % 128 == 0) {
         // Wide B goes to the four-wave kernel: a workgroup per (row tile, slice, 128 columns), up to three resident
         // per CU (768 at once), handed out as earlier ones finish, so more than one round is no loss by itself.
-        // A workgroup alone on its CU needs 1.17 us per tile, 2.1 us when three share the CU; every slab costs
-        // a write and a read of M*N halfs (about 5 TB/s).  Fitted to 36864x9216 at N = 128 / 256.
+        // A tile costs a workgroup 1.4 / 1.8 times as long when two / three share the CU as when it has the CU to
+        // itself; every slab costs a write and a read of M*N halfs.  Fitted to whole-call times of seven of the
+        // reference's weight shapes at N = 128 / 256 and Split_K 1..12: mean 1.6 %, at most 10 % above the best.
         const long   units     = static_cast<long>(m / 128) * (n / 128);
-        const double slab_us   = 4.0 * m * n / 5e6;
+        const double slab_cost = 2.75 * 4.0 * m * n / 5e6;
         int          best      = 1;
         double       best_cost = 1e30;
         for (int s = 1; s <= 32 && s <= kt; s++) {
-            const double wgs      = static_cast<double>(units) * s;
-            const double resident = wgs / 256.0 < 3.0 ? wgs / 256.0 : 3.0;
-            const double rounds   = wgs > 768.0 ? wgs / 768.0 : 1.0;
+            const long   wgs      = units * s;
+            const long   per_cu   = (wgs + 255) / 256 < 3 ? (wgs + 255) / 256 : 3;
+            const double rounds   = wgs > 768 ? std::pow(wgs / 768.0, 0.8) : 1.0;
             const int    longest  = (kt - 1) / s + 1;
-            const double cost     = longest * (1.17 + 0.47 * (resident > 1.0 ? resident - 1.0 : 0.0)) * rounds + (s > 1 ? s * slab_us : 0.0);
+            const double cost     = longest * (1.0 + 0.4 * (per_cu - 1)) * rounds + (s > 1 ? s * slab_cost : 0.0);
             if (cost < best_cost) {
                 best_cost = cost;
                 best      = s;

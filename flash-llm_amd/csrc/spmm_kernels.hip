@@ -420,12 +420,13 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
 //   * all four stream and scatter: round r of a tile gives wave w the 64 vectors (r*4 + w)*64 .. of the
 //     tile's range of Compressed_A; the vectors of the next kAhead tiles are in flight per wave;
 //   * each wave multiplies the whole tile by its own 16*NBW columns: 16 plain 16-byte operand reads
-//     (no clearing: the tile has four readers), 16*NBW MFMAs, B fragments in registers;
+//     (no clearing: the tile has four readers), 16*NBW MFMAs; its B operands are fetched a tile ahead as
+//     whole 128-byte lines and turned into the MFMA layout through LDS (stage_b);
 //   * three tile buffers rotate, so one barrier per tile is enough: in step t a wave reads tile t from one
 //     buffer (complete since the previous barrier), scatters its part of tile t+1 into the second and clears
 //     its quarter of the third (read by everybody before the previous barrier).
-// Every step issues the same number of global loads in the same order (R stream loads and 2*NBW fragment
-// loads, addresses clamped instead of skipped) and every round has all three steps, so the waits the compiler
+// Every step issues the same number of global loads in the same order (R stream loads and 2*NBW loads of B
+// lines, addresses clamped instead of skipped) and every round has all three steps, so the waits the compiler
 // places are exact counts that never drain the stream, and the accumulators stay where they are (with early
 // exits from the unrolled round the register allocation more than doubled).  A tile with more than R*256
 // vectors takes its remaining rounds on a slow path.
@@ -458,15 +459,19 @@ __device__ __forceinline__ void spmm_group_body(uint16_t (&tiles)[3][kTileHalfs]
         for (int rb = 0; rb < 8; rb++)
             acc[nb][rb] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // column col0 + r16 of B; block nb is 16 columns (16 * K halfs) further on (N is a multiple of 128 here)
-    const _Float16* bptr = B + static_cast<size_t>(col0 + (lane & 15)) * K + (lane >> 4) * 8;
+    // B is fetched whole 128-byte lines at a time: load i of a tile takes the 64 k of columns col0 + 8i .. + 7,
+    // eight lanes per column.  (A load of 16 columns x 64 bytes, which is what the MFMA operand layout asks
+    // for, takes twice the requests for the same bytes and measured slower.)  Lane l fetches 16-byte piece
+    // (l % 8) ^ (l / 8) of its column, so that the staging below reads back without bank conflicts.
+    const _Float16* bptr = B + static_cast<size_t>(col0 + (lane >> 3)) * K + (((lane & 7) ^ (lane >> 3)) << 3);
     // operand of this lane inside a 16-row block: row r16 = lane % 16, 16-byte chunk (ks*4 + lane/16) ^ (row%8)
     const int a_off0 = (lane & 15) * (kTileCols * 2) + (((lane >> 4) ^ (lane & 7)) << 4);
     const int a_off1 = a_off0 ^ 64;
 
     uint4 ring[kAhead][R];  // ring[p][r]: this wave's vectors of round r of the tile in slot p
     int   slot_lo[kAhead], slot_n[kAhead];
-    half8 bfrag[2][NBW];
+    uintx4 braw[2 * NBW];  // braw[i]: columns col0 + 8i .. + 7 of B for the next tile, as loaded
+    half8  bfrag[2][NBW];  // the MFMA B operands of the current tile
 
     auto tile_range = [&](int t, int& lo, int& n) {  // tiles at or beyond ke are empty
         const int a = t < ke ? t : ke, b = t + 1 < ke ? t + 1 : ke;
@@ -486,13 +491,29 @@ __device__ __forceinline__ void spmm_group_body(uint16_t (&tiles)[3][kTileHalfs]
             ring[p][r] = load_stream(comp + v);
         }
     };
-    auto load_b = [&](int t) {  // always issued: past the end the last tile's fragments are fetched again
+    auto load_b = [&](int t) {  // always issued: past the end the last tile's lines are fetched again
         const int tc = t < ke ? t : ke - 1;
+#pragma unroll
+        for (int i = 0; i < 2 * NBW; i++)
+            braw[i] = *reinterpret_cast<const uintx4*>(bptr + static_cast<size_t>(i) * 8 * K + tc * kTileCols);
+    };
+    // The lines go to LDS as they are (lane l -> piece l of load i, i.e. column 8i + l/8 at 128 bytes per
+    // column) and are read back at once in the operand layout of the MFMA: lane (r16, g) takes piece
+    // (4*ks + g) ^ (r16 % 8) of column 16*nb + r16.  The 4 KB this needs are the wave's own quarter of the
+    // tile buffer it is about to clear (nobody else touches that quarter between two meetings).  One wave,
+    // in-order LDS: no barrier between write, read and the clearing that follows.
+    // blank: a tile past the slice's end multiplies by zeros, whatever B holds
+    auto stage_b = [&](uint16_t* buf, bool blank) {
+        uintx4* mine = reinterpret_cast<uintx4*>(buf) + wave * (kTileHalfs * 2 / 16 / kGroupWaves);
+        static_assert(2 * NBW * kLanes <= kTileHalfs * 2 / 16 / kGroupWaves, "a wave's B lines must fit its quarter of a tile buffer");
+#pragma unroll
+        for (int i = 0; i < 2 * NBW; i++)
+            mine[i * kLanes + lane] = blank ? uintx4{0u, 0u, 0u, 0u} : braw[i];
 #pragma unroll
         for (int ks = 0; ks < 2; ks++)
 #pragma unroll
             for (int nb = 0; nb < NBW; nb++)
-                bfrag[ks][nb] = *reinterpret_cast<const half8*>(bptr + static_cast<size_t>(nb) * 16 * K + tc * kTileCols + ks * 32);
+                bfrag[ks][nb] = __builtin_bit_cast(half8, mine[(nb * 16 + (lane & 15)) * 8 + ((ks * 4 + (lane >> 4)) ^ (lane & 7))]);
     };
     auto scatter_slot = [&](auto pp, uint16_t* buf) {
         constexpr int p = decltype(pp)::value;
@@ -516,7 +537,7 @@ __device__ __forceinline__ void spmm_group_body(uint16_t (&tiles)[3][kTileHalfs]
             q[i * kLanes + lane] = zero;
     };
     constexpr int kAtOnce = 8;
-    auto          multiply = [&](const uint16_t* buf) {
+    auto          multiply = [&](const half8 (&bf)[2][NBW], const uint16_t* buf) {
         const char* base = reinterpret_cast<const char*>(buf);
 #pragma unroll
         for (int ks = 0; ks < 2; ks++)
@@ -532,7 +553,7 @@ __device__ __forceinline__ void spmm_group_body(uint16_t (&tiles)[3][kTileHalfs]
                     for (int nb = 0; nb < NBW; nb++)
                         // in place (the accumulator is an in/out operand): left to itself the compiler gives the
                         // unrolled steps accumulators of their own and runs out of registers moving between them
-                        asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc[nb][part * kAtOnce + i]) : "v"(a[i]), "v"(bfrag[ks][nb]));
+                        asm("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc[nb][part * kAtOnce + i]) : "v"(a[i]), "v"(bf[ks][nb]));
             }
     };
     // all LDS traffic of this wave has landed, then everybody meets: nothing here waits for global memory
@@ -546,31 +567,25 @@ __device__ __forceinline__ void spmm_group_body(uint16_t (&tiles)[3][kTileHalfs]
     load_b(kb);
     clear_quarter(tiles[0]);
     clear_quarter(tiles[1]);
-    clear_quarter(tiles[2]);
     meet();
     scatter_slot(std::integral_constant<int, 0>{}, tiles[0]);
     request(std::integral_constant<int, 0>{}, kb + kAhead);
+    clear_quarter(tiles[2]);
     meet();
 
-    // step j of a round of three: tile t sits in buffer j and came from slot j.  The MFMAs go first (their
-    // operands have been complete since the last meeting) and run while the wave scatters the next tile; the
-    // next tile's fragments are requested right behind them and have the rest of the step to arrive.
+    // step j of a round of three: tile t sits in buffer j and came from slot j; its B lines were requested a
+    // step ago and go through LDS first.  The MFMAs (their A operands have been complete since the last
+    // meeting) run while the wave requests the next tile's B lines and scatters the next tile.
     // Rounds are always whole: a step past the slice's end finds an empty (all-zero) buffer, scatters nothing,
     // and multiplies zeros by zeros (its fragments are blanked, so that an Inf or NaN in B cannot leak in).
     auto step = [&](auto jj, int t) {
         constexpr int j = decltype(jj)::value, next = (j + 1) % kAhead;
-        if (t >= ke) {
-#pragma unroll
-            for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-                for (int nb = 0; nb < NBW; nb++)
-                    bfrag[ks][nb] = half8{0, 0, 0, 0, 0, 0, 0, 0};
-        }
-        multiply(tiles[j]);
+        stage_b(tiles[(j + 2) % 3], t >= ke);
+        multiply(bfrag, tiles[j]);
         load_b(t + 1);
         scatter_slot(std::integral_constant<int, next>{}, tiles[next]);  // tile t + 1 (empty past the end)
         request(std::integral_constant<int, next>{}, t + 1 + kAhead);
-        clear_quarter(tiles[(j + 2) % 3]);  // tile t - 1, read by all before the last meeting
+        clear_quarter(tiles[(j + 2) % 3]);
         meet();
     };
     for (int t = kb; t < ke; t += kAhead) {

@@ -95,3 +95,27 @@ def test_reduce_closed_form(oracle):
     for i in range(s):
         acc = acc + want[i]
     assert np.array_equal(got, acc.astype(np.float16))
+
+
+def test_slab_page_layout_helper_is_a_bijection_with_known_corners():
+    """The host-side statement of the by-workgroup slab order that the GPU tests lay random slabs out with:
+    a permutation of the S*N*M halfs, and a few entries placed by hand from the layout's description."""
+    from gpu_util import slab_pages, slabs_from_pages
+
+    for m, n, s in [(128, 8, 2), (1024, 16, 7), (1408, 64, 3), (256, 256, 11), (384, 128, 3)]:
+        x = np.arange(s * n * m, dtype=np.int64).reshape(s, n, m)
+        p = slab_pages(x, m, n)
+        assert np.array_equal(np.sort(p), np.arange(s * n * m))
+        assert np.array_equal(slabs_from_pages(p, s, m, n), x)
+    # M = 1024 (8 row tiles = one per XCD), N = 16, S = 7: unit u, slice sl is workgroup sl*8 + u; its 4 KB page starts
+    # at 2048 halfs * workgroup; piece q*64 + g*16 + r = rows 32q+4g.. and 32q+16+4g.. of column r
+    m, n, s = 1024, 16, 7
+    x = np.arange(s * n * m, dtype=np.int64).reshape(s, n, m)
+    p = slab_pages(x, m, n)
+    assert p[0] == x[0, 0, 0] and p[3] == x[0, 0, 3] and p[4] == x[0, 0, 16]
+    assert p[8] == x[0, 1, 0]                                # piece 1: column 1
+    assert p[16 * 8] == x[0, 0, 4]                           # piece 16: g = 1
+    assert p[64 * 8] == x[0, 0, 32]                          # piece 64: q = 1
+    assert p[2048 * 1] == x[0, 0, 128]                       # workgroup 1 = unit 1 (row tile 1), slice 0
+    assert p[2048 * 8] == x[1, 0, 0]                         # workgroup 8 = unit 0, slice 1
+    assert p[2048 * (6 * 8 + 5) + 8 * (2 * 64 + 3 * 16 + 9) + 6] == x[6, 9, 5 * 128 + 64 + 16 + 12 + 2]

@@ -2,7 +2,9 @@
 tables hand-tuned for A100, kernel_benchmark/benchmark.sh:13-15) against its neighbours on the five benchmark shapes:
 the whole SpMM_SplitK_API call at the recommended value may take at most 5 % longer than at the best of
 {s-2 .. s+2}.  Weights are pruned and compressed on the GPU; every timed loop rotates over enough copies of
-Compressed_A that the weights come from HBM; each figure is the median of three loops."""
+Compressed_A that the weights come from HBM; each figure is the median of three loops.
+Two wide-B cases (N a multiple of 128, the four-wave kernel, whose timings step with the number of workgroup
+rounds) are held to 10 %."""
 import sys
 import time
 
@@ -11,7 +13,8 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 
-SHAPES = [(36864, 9216, 16), (9216, 36864, 16), (9216, 9216, 16), (36864, 12288, 32), (49152, 12288, 32)]
+SHAPES = [(36864, 9216, 16, 1.05), (9216, 36864, 16, 1.05), (9216, 9216, 16, 1.05), (36864, 12288, 32, 1.05), (49152, 12288, 32, 1.05),
+          (36864, 9216, 128, 1.10), (9216, 9216, 256, 1.10)]
 
 
 def median_time_us(torch, fn, loops=3, steps=150, settle_s=0.1):
@@ -34,8 +37,8 @@ def median_time_us(torch, fn, loops=3, steps=150, settle_s=0.1):
     return sorted(out)[loops // 2]
 
 
-@pytest.mark.parametrize("m,k,n", SHAPES)
-def test_recommended_split_k_is_within_5_percent_of_its_neighbours(product, m, k, n):
+@pytest.mark.parametrize("m,k,n,bound", SHAPES)
+def test_recommended_split_k_is_within_5_percent_of_its_neighbours(product, m, k, n, bound):
     import torch
 
     assert torch.cuda.is_available()
@@ -57,4 +60,4 @@ def test_recommended_split_k_is_within_5_percent_of_its_neighbours(product, m, k
     for x in cands:
         times[x] = median_time_us(torch, lambda i: product.spmm_splitk(comps[i % copies], offs, b, c, m, n, k, ws, x))
     print("  " + "  ".join(f"{x}: {t:.2f} us" + ("*" if x == s else "") for x, t in times.items()), flush=True)
-    assert times[s] <= 1.05 * min(times.values()), (s, times)
+    assert times[s] <= bound * min(times.values()), (s, times)

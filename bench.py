@@ -99,8 +99,8 @@ def main():
     ap.add_argument("--no-dense", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (rows of A shard with no exchange; "
-                 "see DESIGN.md). Run with --gpus 1.")
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (rows of A would shard across GPUs with no "
+                 "exchange, a split of K adds one all-reduce of C). Run with --gpus 1.")
 
     import numpy as np
     import torch

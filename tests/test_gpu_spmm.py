@@ -391,3 +391,22 @@ def test_decoder_layer_rejects_shapes_that_do_not_chain(product, torch_gpu):
     with pytest.raises(product.HipError) as e:
         layer.forward(x, 16)
     assert e.value.code == 1
+
+
+def test_seeded_random_shapes(product, oracle, torch_gpu):
+    """Forty seeded draws of (M, K, N, Split_K, sparsity) over everything the API dispatches on, including row-tile
+    counts that are no multiple of eight (units beyond whole XCD rounds), slices longer and shorter than the
+    k tiles there are, and both kernels; each against the oracle's product on the same operands."""
+    rng = np.random.default_rng(20240607)
+    for case in range(40):
+        m = 128 * int(rng.integers(1, 14))
+        k = 64 * int(rng.integers(1, 25))
+        n = int(rng.choice([8, 16, 32, 64, 128, 256]))
+        split_k = int(rng.integers(1, min(9, k // 64) + 1))
+        sparsity = float(rng.choice([0.5, 0.7, 0.8, 0.9, 0.97]))
+        say(f"random case {case}: M={m} K={k} N={n} split_k={split_k} sparsity={sparsity}")
+        a = synth.sparse_matrix(m, k, sparsity, 1000 + case)
+        b = synth.dense_b(k, n, 2000 + case)
+        c, _, _ = run_spmm(product, a, b, n, split_k)
+        _, ref = oracle.spmm_model(a, b, n, split_k)
+        assert_close(c, ref, f"case {case}")

@@ -410,3 +410,40 @@ def test_seeded_random_shapes(product, oracle, torch_gpu):
         c, _, _ = run_spmm(product, a, b, n, split_k)
         _, ref = oracle.spmm_model(a, b, n, split_k)
         assert_close(c, ref, f"case {case}")
+
+
+def test_call_can_be_captured_in_a_graph_and_replayed(product, oracle, torch_gpu):
+    """SpMM_SplitK_API allocates nothing and never waits for the host, so a caller may record it into a HIP graph.
+    Replays, with other work and new contents of B between them, must each equal the eager result bit for bit."""
+    torch = torch_gpu
+    say("graph capture")
+    m, n, k, s = 1024, 16, 2048, 5
+    a = synth.sparse_matrix(m, k, 0.8, 31)
+    w = product.SparseWeight(a)
+    b = torch.zeros(n * k, dtype=torch.float16, device="cuda")
+    c = torch.zeros(n * m, dtype=torch.float16, device="cuda")
+    ws = torch.zeros(s * n * m, dtype=torch.float16, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):   # one eager call first, as graph capture wants its kernels loaded already
+        w.matmul(b, n, c=c, workspace=ws, split_k=s, stream=side)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        w.matmul(b, n, c=c, workspace=ws, split_k=s, stream=torch.cuda.current_stream())
+    for rep in range(4):
+        b_h = synth.dense_b(k, n, 40 + rep)
+        b.copy_(torch.from_numpy(b_h).reshape(-1))
+        ws.fill_(float("nan"))
+        c.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = c.cpu().numpy().copy()
+        eager = torch.full((n * m,), float("nan"), dtype=torch.float16, device="cuda")
+        w.matmul(b, n, c=eager, workspace=ws, split_k=s)
+        torch.cuda.synchronize()
+        assert np.array_equal(got.view(np.uint16), eager.cpu().numpy().view(np.uint16)), f"replay {rep}"
+        _, ref = oracle.spmm_model(a, b_h, n, s)
+        assert_close(got.reshape(n, m), ref, f"replay {rep}")

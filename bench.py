@@ -7,7 +7,8 @@ A step is the whole API call (SpMM kernel + split-K reduction) with Compressed_A
 resident in HBM.  Steps rotate over several device copies of Compressed_A (272 MB each, more than the
 256 MB Infinity Cache together) so every launch streams its weights from HBM.
 
-Prints one JSON line; `value` = dense-equivalent TFLOPS = 2*M*N*K / t (the reference's formula,
+Each figure is the median of `--repeats` (5) timed windows of `--steps` calls, with the fastest and slowest
+window beside it.  Prints one JSON line; `value` = dense-equivalent TFLOPS = 2*M*N*K / t (the reference's formula,
 kernel_benchmark/spmm_test.cu:314-316) of the whole call.  `roofline`: `frac` (= `kernel_frac`) is for the
 dominant kernel alone (the SpMM kernel, timed live with events on the launch stream in a second loop
 without the reduction); `whole_call_frac` is the same algorithmic bytes over the time of the whole call,
@@ -86,6 +87,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--settle-ms", type=float, default=300.0,
                     help="untimed run of the same step before the warm-up, so that clocks have left their idle state")
+    ap.add_argument("--repeats", type=int, default=5,
+                    help="timed windows of --steps calls each; the median window is reported, min and max beside it")
     ap.add_argument("--m", type=int, default=36864)
     ap.add_argument("--k", type=int, default=9216)
     ap.add_argument("--n", type=int, default=16)
@@ -154,21 +157,32 @@ def main():
                 i += 1
             torch.cuda.synchronize()
 
-    def timed(fn, steps, warmup):
+    def windows(fn, steps, warmup, repeats):
+        """ms per call of `repeats` timed windows of `steps` back-to-back calls each, after one settle phase and
+        `warmup` untimed calls (the reference times one window of 10 000 launches after 100 warm-ups,
+        kernel_benchmark/spmm_test_utils.h:21-22; several shorter windows show the spread as well)."""
         settle(fn)
         for i in range(warmup):
             fn(i)
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for i in range(steps):
-            fn(i)
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / steps  # ms per call
+        out = []
+        for _ in range(repeats):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(steps):
+                fn(i)
+            e1.record()
+            torch.cuda.synchronize()
+            out.append(e0.elapsed_time(e1) / steps)
+        return sorted(out)
 
-    ms_step = timed(step, args.steps, args.warmup)
-    ms_kernel = timed(kernel_only, args.steps, args.warmup)
+    def timed(fn, steps, warmup):
+        return windows(fn, steps, warmup, 1)[0]
+
+    w_step = windows(step, args.steps, args.warmup, args.repeats)
+    w_kernel = windows(kernel_only, args.steps, args.warmup, args.repeats)
+    ms_step = w_step[len(w_step) // 2]      # the median window is the reported figure
+    ms_kernel = w_kernel[len(w_kernel) // 2]
 
     # correctness of what was just timed (cheap sample of rows against an fp32 product)
     step(0)
@@ -192,6 +206,9 @@ def main():
         "warmup": args.warmup,
         "settle_ms": args.settle_ms,
         "ms_per_step": ms_step,
+        "repeats": args.repeats,
+        "ms_per_step_min": w_step[0],
+        "ms_per_step_max": w_step[-1],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -212,6 +229,8 @@ def main():
             "traffic_source": traffic_source,
             "kernel": "spmm_stream_kernel",
             "kernel_ms": ms_kernel,
+            "kernel_ms_min": w_kernel[0],
+            "kernel_ms_max": w_kernel[-1],
             "kernel_frac": achieved / HBM_PEAK_GBS,
             "whole_call_frac": alg / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "algorithmic_bytes": alg,

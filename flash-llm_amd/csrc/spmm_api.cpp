@@ -174,6 +174,13 @@ int flashllm_device_compress(void* stream, const void* a, int m, int k, const in
     return flashllm_hip_launch_encode(stream, a, m, k, offs, comp);
 }
 
+int flashllm_device_compress_status(void* stream, unsigned int* status)
+{
+    if (!status)
+        return hipErrorInvalidValue;
+    return flashllm_hip_encode_status(stream, status);
+}
+
 size_t flashllm_workspace_bytes(int m, int n, int split_k)
 {
     if (split_k <= 1 || m <= 0 || n <= 0)

@@ -649,12 +649,16 @@ __global__ __launch_bounds__(kGroupThreads, 3) void spmm_group_kernel(const uint
     ke            = ke < kt ? ke : kt;
     const int* toff = offs + static_cast<size_t>(rowtile) * kt;
     _Float16*  o    = pages ? out : out + static_cast<size_t>(slice) * M * N + static_cast<size_t>(rowtile) * kTileRows;
-    // last vector any load of this slice may touch (clamped loads re-read it); vector 0 exists even in an
-    // empty matrix, whose callers allocate at least one
+    // last vector any load of this slice may touch (clamped loads re-read it)
     int vmax = toff[ke] - 1;
     vmax     = vmax > 0 ? vmax : 0;
     // rounds held in registers per tile: two cover 512 vectors (8 KB, tiles up to a quarter full), three 768
     const int whole = offs[static_cast<size_t>(M / kTileRows) * kt];  // vectors in the matrix
+    // An empty matrix has no vector 0: its callers allocate one 4-byte element (reference
+    // kernel_benchmark/spmm_test.cu:258-260).  The always-issued loads then read the first 16 bytes of B
+    // instead (always there, 16-byte aligned); nothing of them is scattered, every tile has zero vectors.
+    if (whole == 0)
+        comp = reinterpret_cast<const uint4*>(B);
     if (whole <= 440LL * (M / kTileRows) * kt)
         spmm_group_body<NBW, 2>(tiles, comp, toff, B, o, M, N, K, kb, ke, col0, vmax, pages);
     else

@@ -4,8 +4,10 @@
 #ifndef FLASHLLM_AMD_SPMM_LAUNCH_H
 #define FLASHLLM_AMD_SPMM_LAUNCH_H
 
-// size of the library-owned slab storage behind flashllm_hip_static_workspace
-#define FLASHLLM_STATIC_WORKSPACE_BYTES (32u << 20)
+#include "flashllm_spmm.h"
+
+// size of the library-owned slab storage behind flashllm_hip_static_workspace: the limit the public header states
+#define FLASHLLM_STATIC_WORKSPACE_BYTES FLASHLLM_STATIC_WORKSPACE_MAX_BYTES
 
 #ifdef __cplusplus
 extern "C" {
@@ -67,6 +69,10 @@ int flashllm_hip_launch_tile_offsets(void* stream, const void* a, int m, int k, 
 
 // out[offs[t]*4 ...] = the packed nonzeros of tile t in the reference's reordered layout.
 int flashllm_hip_launch_encode(void* stream, const void* a, int m, int k, const int* offs, void* out);
+
+// Waits for the stream, then *status = the FLASHLLM_ENCODE_* bits the encoder has recorded on the current device
+// since they were last read, and clears them.
+int flashllm_hip_encode_status(void* stream, unsigned int* status);
 
 #ifdef __cplusplus
 }

@@ -34,6 +34,15 @@ constexpr int kPerBank  = kTileRows * kTileCols / kBanks;  // 256 positions of a
 constexpr int kLanes    = 64;
 constexpr int kMaxFill  = kPerBank + 3;  // at most three padding items
 
+// What the encoder found wrong since the word was last read (FLASHLLM_ENCODE_* bits), one word per GPU.  The host
+// compressor returns an error in these cases; a kernel cannot, so it records them here and carries on.
+__device__ unsigned int g_encode_status;
+
+__device__ __forceinline__ void report(unsigned int what)
+{
+    atomicOr(&g_encode_status, what);
+}
+
 // |x| > 0 in the reference's float compare (csrc/SpMM_API.cu:183): drops +0, -0 and NaN.
 __device__ __forceinline__ bool keeps(uint32_t h)
 {
@@ -184,6 +193,8 @@ __global__ __launch_bounds__(kLanes* kEncodeWaves) void encode_tiles_kernel(cons
                 pad_s[p][0]  = b;
                 pad_s[p][1]  = fill + 1;
                 pad_s[p][2]  = fz < 0 ? 0 : fz;  // the emptiest bank holds fewer than 256 items, so it has a zero
+                if (fz < 0)
+                    report(FLASHLLM_ENCODE_NO_ZERO);
                 fill++;
             }
         }
@@ -224,7 +235,10 @@ __global__ __launch_bounds__(kLanes* kEncodeWaves) void encode_tiles_kernel(cons
     // Never write outside this tile's range of Compressed_A, whatever TileOffsets says: with offsets that were
     // not computed from this very matrix the output is meaningless, but it stays inside the caller's buffer.
     const int room = (offs[t + 1] - offs[t]) * 4;
-    count          = count < room ? count : room;
+    const int full = count;
+    if (room != full && tid == 0)
+        report(FLASHLLM_ENCODE_OFFSETS);
+    count = count < room ? count : room;
     auto      emit     = [&](int b, int h, uint32_t item) {
         const int j = above[h] + __builtin_popcount(reach[h] & ((1u << b) - 1u));
         int       d;
@@ -239,6 +253,8 @@ __global__ __launch_bounds__(kLanes* kEncodeWaves) void encode_tiles_kernel(cons
         }
         if (d >= 0 && d < count)
             out_tile[d] = item;
+        if (d < 0 || d >= full)  // cannot happen while the closed form above is right
+            report(FLASHLLM_ENCODE_RANGE);
     };
 
     for (int bi = 0; bi < kBanksPerWave; bi++) {
@@ -275,6 +291,21 @@ extern "C" int flashllm_hip_launch_tile_offsets(void* stream, const void* a, int
         return static_cast<int>(e);
     hipLaunchKernelGGL(scan_offsets_kernel, dim3(1), dim3(1024), 0, s, offs, tiles);
     return static_cast<int>(hipGetLastError());
+}
+
+extern "C" int flashllm_hip_encode_status(void* stream, unsigned int* status)
+{
+    hipStream_t   s = static_cast<hipStream_t>(stream);
+    unsigned int* word = nullptr;
+    hipError_t    e = hipGetSymbolAddress(reinterpret_cast<void**>(&word), HIP_SYMBOL(g_encode_status));
+    if (e == hipSuccess)
+        e = hipStreamSynchronize(s);
+    if (e == hipSuccess)
+        e = hipMemcpy(status, word, sizeof(unsigned int), hipMemcpyDeviceToHost);
+    const unsigned int zero = 0;
+    if (e == hipSuccess && *status)
+        e = hipMemcpy(word, &zero, sizeof(unsigned int), hipMemcpyHostToDevice);
+    return static_cast<int>(e);
 }
 
 extern "C" int flashllm_hip_launch_encode(void* stream, const void* a, int m, int k, const int* offs, void* out)

@@ -47,6 +47,7 @@ SIGNATURES = {
     "flashllm_splitk_reduce": (ctypes.c_int, [_vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "flashllm_device_tile_offsets": (ctypes.c_int, [_vp, _vp, ctypes.c_int, ctypes.c_int, _vp, ctypes.POINTER(ctypes.c_longlong)]),
     "flashllm_device_compress": (ctypes.c_int, [_vp, _vp, ctypes.c_int, ctypes.c_int, _vp, _vp]),
+    "flashllm_device_compress_status": (ctypes.c_int, [_vp, ctypes.POINTER(ctypes.c_uint)]),
     "flashllm_splitk_heuristic": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "flashllm_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "flashllm_decoder_layer_linears": (ctypes.c_int, [_vp, ctypes.POINTER(DecoderLayerStruct), _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp]),
@@ -216,11 +217,24 @@ def device_compress(a_dev, stream=None):
     rc = lib().flashllm_device_tile_offsets(_stream(stream), _ptr(a_dev), m, k, _ptr(offs), ctypes.byref(nnz))
     if rc:
         raise CompressError(rc) if rc < 0 else HipError(rc)
-    comp = torch.empty(max(int(nnz.value), 4), dtype=torch.int32, device=a_dev.device)
+    comp = torch.empty(max(int(nnz.value), 1), dtype=torch.int32, device=a_dev.device)
     rc = lib().flashllm_device_compress(_stream(stream), _ptr(a_dev), m, k, _ptr(offs), _ptr(comp))
     if rc:
         raise CompressError(rc) if rc < 0 else HipError(rc)
     return comp[: int(nnz.value)], offs
+
+
+ENCODE_NO_ZERO, ENCODE_OFFSETS, ENCODE_RANGE = 1, 2, 4  # FLASHLLM_ENCODE_*
+
+
+def device_compress_status(stream=None):
+    """flashllm_device_compress_status: waits for the stream and returns (and clears) the FLASHLLM_ENCODE_* bits
+    the device encoder has recorded on the current GPU; 0 = nothing wrong."""
+    word = ctypes.c_uint(0)
+    rc = lib().flashllm_device_compress_status(_stream(stream), ctypes.byref(word))
+    if rc:
+        raise HipError(rc)
+    return int(word.value)
 
 
 class SparseWeight:
@@ -238,7 +252,7 @@ class SparseWeight:
         self.nnz = items.size
         self.num_offsets = offsets.size
         if items.size == 0:  # fully sparse: keep one addressable element, as the reference's callers do
-            items = np.zeros(4, dtype=np.uint32)
+            items = np.zeros(1, dtype=np.uint32)
         self.comp = torch.from_numpy(items.view(np.int32)).to(device)
         self.offs = torch.from_numpy(offsets).to(device)
         self.split_k = split_k

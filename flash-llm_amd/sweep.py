@@ -51,7 +51,7 @@ def run_case(torch, name, a, n, split_k=None, b_dist="normal", dense=True, copie
     items, offsets = F.init_sparse_matrix_a(a)
     nnz = int(items.size)
     copies = copies or max(1, min(4, int(1.2e9 // max(1, 4 * nnz))))
-    comps = [torch.from_numpy(items.view(np.int32) if nnz else np.zeros(4, np.int32)).cuda() for _ in range(copies)]
+    comps = [torch.from_numpy(items.view(np.int32) if nnz else np.zeros(1, np.int32)).cuda() for _ in range(copies)]
     offs = torch.from_numpy(offsets).cuda()
     b_h = synth.dense_b(k, n, 1, dist=b_dist)
     b = torch.from_numpy(b_h).cuda()

@@ -153,11 +153,27 @@ int flashllm_splitk_heuristic(int M, int N, int K);
  * what flashllm_device_tile_offsets computed for this very A: the encoder
  * trusts them for where each tile goes.  With other offsets the contents of
  * Compressed_A are unspecified; the encoder still never writes outside
- * [TileOffsets[t], TileOffsets[t+1]) for tile t, and there is no error code
- * for it (the call is asynchronous).
+ * [TileOffsets[t], TileOffsets[t+1]) for tile t; the call is asynchronous, so
+ * the mismatch is reported by flashllm_device_compress_status afterwards.
  */
 int flashllm_device_tile_offsets(void* stream, const void* A, int M, int K, int* TileOffsets, long long* NNZ_padded);
 int flashllm_device_compress(void* stream, const void* A, int M, int K, const int* TileOffsets, void* Compressed_A);
+
+/*
+ * What flashllm_device_compress found wrong, for callers that want the host compressor's error behaviour from the
+ * asynchronous device one: waits for the stream, stores in *Status the bits recorded on the current GPU since the
+ * last call of this function (0 = every tile was encoded as the host compressor would), and clears them.
+ *  FLASHLLM_ENCODE_NO_ZERO  a padding item was needed in a bank without a zero position (the host compressor
+ *                           returns FLASHLLM_E_NOZERO, the reference asserts, csrc/SpMM_API.cu:282);
+ *  FLASHLLM_ENCODE_OFFSETS  TileOffsets did not belong to this matrix: some tile's range differs from its count
+ *                           (items beyond the range were dropped, a longer range was left partly unwritten);
+ *  FLASHLLM_ENCODE_RANGE    an item's computed place lay outside its tile (an internal error; the item was dropped).
+ * Returns 0 or a hipError_t value.
+ */
+#define FLASHLLM_ENCODE_NO_ZERO 1u
+#define FLASHLLM_ENCODE_OFFSETS 2u
+#define FLASHLLM_ENCODE_RANGE 4u
+int flashllm_device_compress_status(void* stream, unsigned int* Status);
 
 /* Bytes the caller must provide as Reduction_Workspace (0 when Split_K == 1);
  * the contract of reference build/SpMM_API.cuh:33-36. */

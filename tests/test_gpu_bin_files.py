@@ -24,7 +24,7 @@ def load_and_multiply(product, names, m, k, b_host, n, split_k):
         offsets = np.frombuffer(f.read(4 * num_offsets), dtype=np.int32)
     assert items.size == nnz and offsets.size == num_offsets
     # a fully sparse weight has no items: the callers allocate at least one element (kernel_benchmark/spmm_test.cu:258-259)
-    comp = torch.zeros(max(nnz, 4), dtype=torch.int32, device="cuda")
+    comp = torch.zeros(max(nnz, 1), dtype=torch.int32, device="cuda")
     comp[:nnz] = torch.from_numpy(items.copy())
     offs = torch.from_numpy(offsets.copy()).cuda()
     b = torch.from_numpy(b_host).cuda()

@@ -40,6 +40,7 @@ def check_against_oracle(product, oracle, torch, a, what):
     assert items.shape == want_items.shape, f"{what}: {items.shape} vs {want_items.shape}"
     bad = np.flatnonzero(items != want_items)
     assert bad.size == 0, f"{what}: {bad.size} items differ, first at {bad[:4]}"
+    assert product.device_compress_status() == 0, f"{what}: the encoder recorded an error"
 
 
 def test_config1(product, oracle, torch_gpu):
@@ -119,6 +120,28 @@ def test_spmm_on_device_compressed_weights(product, oracle, torch_gpu):
     torch.cuda.synchronize()
     _, ref = oracle.spmm_model(a, b, n, 4)
     assert_close(c.cpu().numpy().reshape(n, m), ref, "spmm on device-compressed weights")
+
+
+def test_status_reports_offsets_of_another_matrix(product, torch_gpu):
+    """The encoder trusts TileOffsets for where a tile goes.  Given those of a different matrix it stays inside
+    each tile's range, finishes normally, and says so through flashllm_device_compress_status; the word is
+    cleared by reading it."""
+    torch = torch_gpu
+    say("device compress: status word")
+    a = torch.from_numpy(synth.sparse_matrix(256, 128, 0.8, 31)).cuda()
+    other = torch.from_numpy(synth.sparse_matrix(256, 128, 0.7, 32)).cuda()
+    comp, offs = product.device_compress(a)
+    assert product.device_compress_status() == 0
+    _, offs_other = product.device_compress(other)
+    assert product.device_compress_status() == 0
+    out = torch.zeros(int(offs_other[-1].item()) * 4, dtype=torch.int32, device="cuda")
+    rc = product.lib().flashllm_device_compress(None, a.data_ptr(), 256, 128, offs_other.data_ptr(), out.data_ptr())
+    assert rc == 0
+    assert product.device_compress_status() == product.ENCODE_OFFSETS
+    assert product.device_compress_status() == 0
+    # and the right offsets still give the right bytes afterwards
+    again, _ = product.device_compress(a)
+    assert torch.equal(again, comp) and product.device_compress_status() == 0
 
 
 def test_rejects_bad_arguments(product, torch_gpu):

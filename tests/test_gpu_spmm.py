@@ -128,22 +128,46 @@ def test_wide_b_ragged_tiles_and_empty_slices(product, oracle, torch_gpu):
         assert_close(c, ref, f"wide ragged split_k={split_k}")
 
 
-def test_wide_b_matches_the_narrow_kernel_bit_for_bit(product, torch_gpu):
+@pytest.mark.parametrize("n,sparsity", [(128, 0.8), (256, 0.8), (256, 0.6)])
+def test_wide_b_matches_the_narrow_kernel_bit_for_bit(product, torch_gpu, n, sparsity):
     """Both kernels accumulate a slice's k tiles in order with the same MFMA, so their slabs are identical:
-    the 128 columns of a wide call equal two 64-column calls on the column halves."""
+    the columns of a wide call equal 64-column calls on its column groups.  At 60 % sparsity the wide kernel
+    holds three rounds of a tile in registers instead of two (its other instantiation)."""
     torch = torch_gpu
-    say("wide B vs narrow kernel")
-    m, k, n, s = 1024, 2048, 128, 4
-    a = synth.sparse_matrix(m, k, 0.8, 46, dist="normal", sigma=0.05)
+    say(f"wide B vs narrow kernel n={n} sparsity={sparsity}")
+    m, k, s = 1024, 2048, 4
+    a = synth.sparse_matrix(m, k, sparsity, 46, dist="normal", sigma=0.05)
     b_h = synth.dense_b(k, n, 47, dist="normal")
     wide, w, _ = run_spmm(product, a, b_h, n, s)
     b = torch.from_numpy(b_h).cuda()
-    for half in range(2):
+    for part in range(n // 64):
         c = torch.empty(64 * m, dtype=torch.float16, device="cuda")
         ws = torch.empty(s * 64 * m, dtype=torch.float16, device="cuda")
-        product.spmm_splitk(w.comp, w.offs, b[half * 64:(half + 1) * 64].contiguous(), c, m, 64, k, ws, s)
+        product.spmm_splitk(w.comp, w.offs, b[part * 64:(part + 1) * 64].contiguous(), c, m, 64, k, ws, s)
         torch.cuda.synchronize()
-        assert np.array_equal(c.cpu().numpy().view(np.uint16), wide[half * 64:(half + 1) * 64].reshape(-1).view(np.uint16))
+        assert np.array_equal(c.cpu().numpy().view(np.uint16), wide[part * 64:(part + 1) * 64].reshape(-1).view(np.uint16))
+
+
+@pytest.mark.parametrize("n", [16, 64, 128])
+def test_empty_matrix_with_a_four_byte_allocation(product, torch_gpu, n):
+    """A matrix without nonzeros has no items; the reference's callers then allocate a single 4-byte element
+    (kernel_benchmark/spmm_test.cu:258-260).  No kernel may count on more."""
+    torch = torch_gpu
+    say(f"empty matrix, one-element Compressed_A, n={n}")
+    m, k = 512, 1024
+    a = np.zeros((m, k), dtype=np.float16)
+    items, offsets = product.init_sparse_matrix_a(a)
+    assert items.size == 0 and not offsets.any()
+    comp = torch.zeros(1, dtype=torch.int32, device="cuda")
+    assert comp.numel() * comp.element_size() == 4
+    offs = torch.from_numpy(offsets).cuda()
+    b = torch.from_numpy(synth.dense_b(k, n, 48)).cuda()
+    for split_k in (1, 3):
+        c = torch.full((n * m,), float("nan"), dtype=torch.float16, device="cuda")
+        ws = torch.full((split_k * n * m,), float("nan"), dtype=torch.float16, device="cuda")
+        product.spmm_splitk(comp, offs, b, c, m, n, k, ws, split_k)
+        torch.cuda.synchronize()
+        assert not c.cpu().numpy().view(np.uint16).any()
 
 
 def test_ones_matrix_subset_sums(product, oracle, torch_gpu):

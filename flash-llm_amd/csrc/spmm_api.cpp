@@ -40,13 +40,27 @@ bool known_order(int slab_order)
     return slab_order == FLASHLLM_SLABS_PLAIN || slab_order == FLASHLLM_SLABS_BY_WORKGROUP;
 }
 
-int launch_partials(void* stream, const void* comp, const int* offs, const void* b, void* c, int m, int n, int k, void* ws, int split_k, int slab_order)
+int launch_partials(void* stream, const void* comp, const int* offs, const void* b, int ldb, void* c, int m, int n, int k, void* ws, int split_k, int slab_order)
 {
     const int pages = slab_order == FLASHLLM_SLABS_BY_WORKGROUP;
     // wide B: four waves share every scattered tile; otherwise one wave per (row tile, slice, column group)
     if (n % 128 == 0)
-        return flashllm_hip_launch_spmm_group(stream, comp, offs, b, split_k == 1 ? c : ws, m, n, k, split_k, pages);
-    return flashllm_hip_launch_spmm(stream, comp, offs, b, split_k == 1 ? c : ws, m, n, k, split_k, pages);
+        return flashllm_hip_launch_spmm_group(stream, comp, offs, b, ldb, split_k == 1 ? c : ws, m, n, k, split_k, pages);
+    return flashllm_hip_launch_spmm(stream, comp, offs, b, ldb, split_k == 1 ? c : ws, m, n, k, split_k, pages);
+}
+
+// SpMM_SplitK_API with B's columns ldb halfs apart (the public entry points take a dense column-major B: ldb = K)
+int spmm_splitk_ldb(void* stream, const void* comp, const int* offs, const void* b, int ldb, void* c, int m, int n, int k, void* ws, int split_k)
+{
+    int rc = check_shape(comp, offs, b, c, m, n, k, ws, split_k);
+    if (rc)
+        return rc;
+    if (ldb < k || ldb % 8)
+        return hipErrorInvalidValue;
+    rc = launch_partials(stream, comp, offs, b, ldb, c, m, n, k, ws, split_k, FLASHLLM_SLABS_BY_WORKGROUP);
+    if (rc || split_k == 1)
+        return rc;
+    return flashllm_hip_launch_reduce_pages(stream, c, ws, m, n, split_k, 0);
 }
 
 // The reduction behind launch_partials with the same slab_order.
@@ -78,7 +92,7 @@ int flashllm_spmm_partials(void*       stream,
         return bad;
     if (!known_order(slab_order))
         return hipErrorInvalidValue;
-    return launch_partials(stream, comp, offs, b, c, m, n, k, ws, split_k, slab_order);
+    return launch_partials(stream, comp, offs, b, k, c, m, n, k, ws, split_k, slab_order);
 }
 
 int flashllm_splitk_reduce(void* stream, void* c, const void* ws, int m, int n, int split_k, int slab_order)
@@ -260,7 +274,7 @@ int flashllm_decoder_layer_linears(void*                         stream,
                                    int                           tokens,
                                    void*                         ws)
 {
-    if (!layer || !x || !qkv_out || !attn_in || !attn_out || !ffn_mid || !y)
+    if (!layer || !x || !qkv_out || !attn_out || !ffn_mid || !y)
         return hipErrorInvalidValue;
     const flashllm_sparse_weight& q = layer->qkv;
     const flashllm_sparse_weight& o = layer->attn_out;
@@ -274,16 +288,20 @@ int flashllm_decoder_layer_linears(void*                         stream,
             return 1;
         return w.split_k > 0 ? w.split_k : flashllm_splitk_heuristic(w.m, tokens, w.k);
     };
-    auto linear = [&](const flashllm_sparse_weight& w, const void* in, void* out, int limit) {
-        return flashllm_spmm_splitk(stream, nullptr, w.nz_weights, w.tile_offsets, in, out, w.m, tokens, w.k, ws, split(w, limit));
+    auto linear = [&](const flashllm_sparse_weight& w, const void* in, int ld_in, void* out, int limit) {
+        return spmm_splitk_ldb(stream, w.nz_weights, w.tile_offsets, in, ld_in, out, w.m, tokens, w.k, ws, split(w, limit));
     };
-    int rc = linear(q, x, qkv_out, 64);
+    int rc = linear(q, x, hidden, qkv_out, 64);
     if (rc)
         return rc;
-    rc = flashllm_hip_launch_take_rows(stream, attn_in, qkv_out, hidden, tokens, q.m);
-    if (rc)
-        return rc;
-    rc = linear(o, attn_in, attn_out, 64);
+    // The attention-output linear multiplies the first `hidden` rows of every column of qkv_out: it reads them
+    // where they are (columns q.m halfs apart).  A caller that also wants them contiguous passes attn_in.
+    if (attn_in) {
+        rc = flashllm_hip_launch_take_rows(stream, attn_in, qkv_out, hidden, tokens, q.m);
+        if (rc)
+            return rc;
+    }
+    rc = linear(o, qkv_out, q.m, attn_out, 64);
     if (rc)
         return rc;
     // FFN1 with the ReLU folded into its reduction when there is one
@@ -295,7 +313,7 @@ int flashllm_decoder_layer_linears(void*                         stream,
                 : flashllm_hip_launch_relu(stream, ffn_mid, static_cast<long>(f1.m) * tokens);
     if (rc)
         return rc;
-    return linear(f2, ffn_mid, y, 128);
+    return linear(f2, ffn_mid, f2.k, y, 128);
 }
 
 }  // extern "C"

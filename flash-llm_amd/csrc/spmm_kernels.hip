@@ -219,33 +219,76 @@ __device__ __forceinline__ void take_16_and_wait(uintx4 (&a0)[8], uintx4 (&a1)[8
         : "memory");
 }
 
-// NB: 16-column blocks per wave (1 for N <= 16, 2 for N = 32, 4 for N >= 64).
-// DEPTH: ring slots = 1 KB chunks in flight per wave (8; 6 at NB = 4, which keeps that instance within
-// 256 VGPRs = two waves per SIMD).
-template<int NB, int DEPTH>
-__global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __restrict__ comp,
-                                                            const int* __restrict__ offs,
-                                                            const _Float16* __restrict__ B,
-                                                            _Float16* __restrict__ out,
-                                                            int M,
-                                                            int N,
-                                                            int K,
-                                                            int split_k,
-                                                            int col_groups,
-                                                            int pages)
+// One 1 KB piece of B (eight columns x the 64 k of a k tile, i.e. eight whole 128-byte lines) from global memory
+// straight into LDS, without passing through registers: lane l delivers its 16 bytes at lds + 16*l.  The wave's
+// vector-memory counter counts it like any load; the compiler does not know of it.
+__device__ __forceinline__ void load_to_lds_16(const void* src, uint32_t lds)
 {
-    __shared__ __attribute__((aligned(16))) uint16_t tile[kTileHalfs];
+    uint32_t saved;
+    asm volatile(
+        "s_mov_b32 %0, m0\n\t"
+        "s_mov_b32 m0, %2\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %1, off\n\t"
+        "s_mov_b32 m0, %0"
+        : "=&s"(saved)
+        : "v"(src), "s"(lds)
+        : "memory");
+}
 
-    const int lane = threadIdx.x;
+// NB: 16-column blocks per wave (1 for N <= 16, 2 for N = 32, 4 for N >= 64).
+// DEPTH: ring slots = 1 KB chunks in flight per wave.
+// W: waves per workgroup.  W == 1: a wave is a workgroup and fetches its own B fragments from L2.
+//
+// W > 1 (N = 32 and 64, where the 2*NB fragment loads per tile and wave are what holds the one-wave form back):
+// the W waves of a workgroup take the SAME K slice of W consecutive row tiles, so they need the same B, and B
+// is staged in LDS once per workgroup, as the reference stages one B tile per thread block for all of its
+// warps (csrc/MatMulUtilities.cuh:39-75).  Every wave keeps its private tile and its own stream and runs
+// freely; the waves meet once per window of G k tiles:
+//   * the window's B (G k tiles x 16*NB columns x 128 bytes) is fetched as whole 128-byte lines by
+//     load_to_lds_16, each wave two of the window's 1 KB pieces; piece (l % 8) ^ (l / 8) of a line goes to
+//     slot l % 8 of its column, so the operand reads below are free of bank conflicts;
+//   * two windows of LDS alternate.  Before a wave reads the first fragment of window w it makes sure its own
+//     pieces of w have landed (they were requested a whole window earlier: after DEPTH younger ring loads the
+//     ring's own waits have already covered them, otherwise it drains) and meets the others at a barrier;
+//     past the barrier everybody has finished reading window w-1, whose LDS then receives window w+1;
+//   * a tile's fragments are 2*NB plain 16-byte LDS reads issued with the operand exchanges.
+// A wave without nonzeros in the slice, or beyond the last row tile, still fetches its pieces and attends
+// every barrier.
+template<int NB, int DEPTH, int W, int G>
+__global__ __launch_bounds__(kLanes* W) void spmm_stream_kernel(const uint4* __restrict__ comp,
+                                                                const int* __restrict__ offs,
+                                                                const _Float16* __restrict__ B,
+                                                                int ldb,
+                                                                _Float16* __restrict__ out,
+                                                                int M,
+                                                                int N,
+                                                                int K,
+                                                                int split_k,
+                                                                int col_groups,
+                                                                int pages)
+{
+    constexpr int kBTile  = NB * 2048;                     // bytes of B per k tile in LDS: 16*NB columns x 128
+    constexpr int kBBytes = W > 1 ? 2 * G * kBTile : 0;    // two windows
+    constexpr int kPieces = W > 1 ? G * 2 * NB / W : 0;    // 1 KB pieces of a window each wave fetches
+    static_assert(W == 1 || (G * 2 * NB) % W == 0, "the pieces of a window must divide among the waves");
+    static_assert((G & (G - 1)) == 0, "G must be a power of two");
+    // the windows of B first (the LDS address of a direct load travels in M0 and stays small), then the waves' tiles
+    __shared__ __attribute__((aligned(16))) unsigned char lds[kBBytes + W * kTileHalfs * 2];
+
+    const int lane = threadIdx.x & (kLanes - 1);
+    const int wave = W > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x / kLanes) : 0;
+    uint16_t* const tile = reinterpret_cast<uint16_t*>(lds + kBBytes) + wave * kTileHalfs;
     const int r16  = lane & 15;  // row inside a 16-row block / output column
     const int g    = lane >> 4;  // which 8-wide k chunk of a 32-wide k step
     const int kt   = K / kTileCols;
-    // unit = (row tile, column group), column group fastest: the column groups of a row tile read the
-    // same weights and meet in one L2
+    // W == 1: unit = (row tile, column group), column group fastest: the column groups of a row tile read the
+    // same weights and meet in one L2.  W > 1: unit = W consecutive row tiles, all 16*NB columns.
     int unit, slice;
     unit_of_workgroup(blockIdx.x, gridDim.x / split_k, split_k, unit, slice);
-    const int rowtile = unit / col_groups;
-    const int col0    = (unit % col_groups) * (16 * NB);
+    const int  rowtile   = W > 1 ? unit * W + wave : unit / col_groups;
+    const int  col0      = W > 1 ? 0 : (unit % col_groups) * (16 * NB);
+    const bool have_rows = W == 1 || rowtile < M / kTileRows;
     // HW_ID.wave_id: which of the SIMD's wave slots this wave sits in (bit 0 tells the two apart)
     const int wave_slot = __builtin_amdgcn_s_getreg(4 | (0 << 6) | (3 << 11)) & 1;
 
@@ -263,9 +306,42 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
         for (int rb = 0; rb < 8; rb++)
             acc[nb][rb] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    const int* toff = offs + static_cast<size_t>(rowtile) * kt;
+    const int* toff = offs + static_cast<size_t>(have_rows ? rowtile : 0) * kt;
     const int  vbeg = toff[kb];
-    const int  vend = toff[ke];
+    const int  vend = have_rows ? toff[ke] : vbeg;
+
+    // ---- the shared B windows (W > 1 only) ----
+    const uint32_t bwin_lds = lds_offset(&lds[0]);
+    int            since    = 0;  // ring loads this wave has issued since it last requested pieces of B
+    // this wave's pieces of window w: piece j is k tile j / (2*NB) of the window, columns 8*(j % (2*NB)) .. +7
+    auto fetch_window = [&](int w) {
+#pragma unroll
+        for (int i = 0; i < kPieces; i++) {
+            const int j  = wave * kPieces + i;
+            int       tk = kb + w * G + j / (2 * NB);
+            tk           = tk < ke ? tk : ke - 1;  // past the slice's end: any valid lines, nobody reads them
+            const int c  = 8 * (j % (2 * NB)) + (lane >> 3);
+            load_to_lds_16(B + static_cast<size_t>(c) * ldb + tk * kTileCols + (((lane & 7) ^ (lane >> 3)) << 3),
+                           bwin_lds + (w & 1) * (G * kBTile) + j * 1024);
+        }
+        since = 0;
+    };
+    // before the first read of window w
+    auto open_window = [&](int w) {
+        // At most DEPTH loads still in flight: with DEPTH ring loads younger than this wave's pieces of window w
+        // those have landed (loads complete in order); the ring itself is rarely touched by this wait, a slot is
+        // only refilled after the wait for its previous contents.  With fewer younger loads: drain.
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DEPTH) : "memory");
+        if (since < DEPTH)
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        asm volatile("s_barrier" ::: "memory");
+        if (kb + (w + 1) * G < ke)
+            fetch_window(w + 1);
+    };
+    if constexpr (W > 1) {
+        if (kb < ke)
+            fetch_window(0);
+    }
 
     if (vend > vbeg) {
         // operand addresses: row r16 of a row block, 16-byte chunk (ks*4+g) ^ (row%8)
@@ -276,22 +352,31 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
         for (int nb = 0; nb < NB; nb++) {
             int n    = col0 + nb * 16 + r16;
             n        = n < N ? n : N - 1;  // N == 8: lanes 8..15 compute columns nobody stores
-            bptr[nb] = B + static_cast<size_t>(n) * K + g * 8;
+            bptr[nb] = B + static_cast<size_t>(n) * ldb + g * 8;
         }
-        const uint32_t tile_lds = lds_offset(&tile[0]);
+        const uint32_t tile_lds = lds_offset(tile);
         uint32_t       a_addr0[8], a_addr1[8];  // LDS byte addresses of this lane's operands: k step 0 / 1 of row block rb
 #pragma unroll
         for (int rb = 0; rb < 8; rb++) {
             a_addr0[rb] = tile_lds + rb * (16 * kTileCols * 2) + a_off0;
             a_addr1[rb] = tile_lds + rb * (16 * kTileCols * 2) + a_off1;
         }
-        half8          bfrag[2][NB];  // B fragments of the open tile
+        half8          bfrag[2][NB];  // B fragments of the open tile (W == 1) / of the tile being multiplied
         auto           load_b = [&](int t) {
 #pragma unroll
             for (int ks = 0; ks < 2; ks++)
 #pragma unroll
                 for (int nb = 0; nb < NB; nb++)
                     bfrag[ks][nb] = *reinterpret_cast<const half8*>(bptr[nb] + t * kTileCols + ks * 32);
+        };
+        // W > 1: the fragments of k step ks of tile t out of its window: column 16*nb + r16 holds piece
+        // (4*ks + g) at slot (4*ks + g) ^ (r16 % 8), the same offsets as an operand of A inside a row block
+        auto read_b = [&](int t, int ks) {
+            const int            i    = t - kb;
+            const unsigned char* base = lds + ((i / G) & 1) * (G * kBTile) + (i % G) * kBTile + (ks ? a_off1 : a_off0);
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++)
+                bfrag[ks][nb] = *reinterpret_cast<const half8*>(base + nb * 2048);
         };
 
         clear_tile(tile, lane);
@@ -305,7 +390,8 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
             ring[d] = uint4{0u, 0u, 0u, 0u};
 
         int t = kb, tile_lo = vbeg, tile_hi = toff[kb + 1], next_hi = toff[kb + 2];
-        load_b(t);
+        if constexpr (W == 1)
+            load_b(t);
 
         // Chunks -DEPTH .. -1 only fill the ring: none of their lanes reaches tile_lo, and a tile can
         // only "end" there when it is empty.
@@ -319,6 +405,10 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                     if (v >= tile_lo && v < tile_hi)
                         scatter_vector(tile, cur);
                     while (tile_hi <= ve) {  // a tile ends inside, or exactly at the end of, this chunk
+                        if constexpr (W > 1) {
+                            if (((t - kb) & (G - 1)) == 0)
+                                open_window((t - kb) / G);
+                        }
                         if (tile_hi > tile_lo) {
                             // NB <= 2: all 16 operands in one batch.  NB == 4: one 32-wide k step at a time, which
                             // keeps the kernel within 256 VGPRs (two waves per SIMD).
@@ -326,6 +416,8 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
 #pragma unroll
                                 for (int ks = 0; ks < 2; ks++) {
                                     uintx4 a[8];
+                                    if constexpr (W > 1)
+                                        read_b(t, ks);
                                     take_8_and_wait(a, ks ? a_addr1 : a_addr0);
 #pragma unroll
                                     for (int rb = 0; rb < 8; rb++)
@@ -337,6 +429,10 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                             }
                             else {
                                 uintx4 a0[8], a1[8];
+                                if constexpr (W > 1) {
+                                    read_b(t, 0);
+                                    read_b(t, 1);
+                                }
                                 take_16_and_wait(a0, a1, a_addr0, a_addr1);
 #pragma unroll
                                 for (int rb = 0; rb < 8; rb++)
@@ -368,7 +464,8 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                         else
                             __builtin_amdgcn_s_setprio(0);
                         if (t < ke) {
-                            load_b(t);
+                            if constexpr (W == 1)
+                                load_b(t);
                             tile_hi = next_hi;
                             next_hi = toff[t + 2];
                             if (v >= tile_lo && v < tile_hi)  // the rest of this chunk opens the next tile
@@ -384,14 +481,23 @@ __global__ __launch_bounds__(kLanes) void spmm_stream_kernel(const uint4* __rest
                     int vn  = v + DEPTH * kLanes;
                     vn      = vn < vlast ? vn : vlast;
                     ring[d] = load_stream(comp + vn);
+                    if constexpr (W > 1)
+                        since++;
                 }
             }
         }
     }
+    else if constexpr (W > 1) {
+        // nothing to multiply: this wave's part in the windows remains
+        for (int w = 0; w * G < ke - kb; w++)
+            open_window(w);
+    }
 
+    if (!have_rows)
+        return;
     // D layout of the 16x16 MFMA: lane holds column r16, rows 4*g .. 4*g+3 of each 16-row block.
-    if (pages) {
-        store_pages<NB>(out, acc, 0, N, lane);
+    if (pages) {  // a workgroup's pages: wave by wave, NB each
+        store_pages<NB>(out, acc, wave * NB, N, lane);
         return;
     }
     _Float16* o = out + static_cast<size_t>(slice) * M * N + static_cast<size_t>(rowtile) * kTileRows + g * 4;
@@ -439,6 +545,7 @@ __device__ __forceinline__ void spmm_group_body(uint16_t (&tiles)[3][kTileHalfs]
                                                 const uint4* __restrict__ comp,
                                                 const int* __restrict__ toff,
                                                 const _Float16* __restrict__ B,
+                                                int ldb,
                                                 _Float16* __restrict__ o,
                                                 int M,
                                                 int N,
@@ -463,7 +570,7 @@ __device__ __forceinline__ void spmm_group_body(uint16_t (&tiles)[3][kTileHalfs]
     // eight lanes per column.  (A load of 16 columns x 64 bytes, which is what the MFMA operand layout asks
     // for, takes twice the requests for the same bytes and measured slower.)  Lane l fetches 16-byte piece
     // (l % 8) ^ (l / 8) of its column, so that the staging below reads back without bank conflicts.
-    const _Float16* bptr = B + static_cast<size_t>(col0 + (lane >> 3)) * K + (((lane & 7) ^ (lane >> 3)) << 3);
+    const _Float16* bptr = B + static_cast<size_t>(col0 + (lane >> 3)) * ldb + (((lane & 7) ^ (lane >> 3)) << 3);
     // operand of this lane inside a 16-row block: row r16 = lane % 16, 16-byte chunk (ks*4 + lane/16) ^ (row%8)
     const int a_off0 = (lane & 15) * (kTileCols * 2) + (((lane >> 4) ^ (lane & 7)) << 4);
     const int a_off1 = a_off0 ^ 64;
@@ -495,7 +602,7 @@ __device__ __forceinline__ void spmm_group_body(uint16_t (&tiles)[3][kTileHalfs]
         const int tc = t < ke ? t : ke - 1;
 #pragma unroll
         for (int i = 0; i < 2 * NBW; i++)
-            braw[i] = *reinterpret_cast<const uintx4*>(bptr + static_cast<size_t>(i) * 8 * K + tc * kTileCols);
+            braw[i] = *reinterpret_cast<const uintx4*>(bptr + static_cast<size_t>(i) * 8 * ldb + tc * kTileCols);
     };
     // The lines go to LDS as they are (lane l -> piece l of load i, i.e. column 8i + l/8 at 128 bytes per
     // column) and are read back at once in the operand layout of the MFMA: lane (r16, g) takes piece
@@ -627,6 +734,7 @@ template<int NBW>
 __global__ __launch_bounds__(kGroupThreads, 3) void spmm_group_kernel(const uint4* __restrict__ comp,
                                                                   const int* __restrict__ offs,
                                                                   const _Float16* __restrict__ B,
+                                                                  int ldb,
                                                                   _Float16* __restrict__ out,
                                                                   int M,
                                                                   int N,
@@ -660,9 +768,9 @@ __global__ __launch_bounds__(kGroupThreads, 3) void spmm_group_kernel(const uint
     if (whole == 0)
         comp = reinterpret_cast<const uint4*>(B);
     if (whole <= 440LL * (M / kTileRows) * kt)
-        spmm_group_body<NBW, 2>(tiles, comp, toff, B, o, M, N, K, kb, ke, col0, vmax, pages);
+        spmm_group_body<NBW, 2>(tiles, comp, toff, B, ldb, o, M, N, K, kb, ke, col0, vmax, pages);
     else
-        spmm_group_body<NBW, 3>(tiles, comp, toff, B, o, M, N, K, kb, ke, col0, vmax, pages);
+        spmm_group_body<NBW, 3>(tiles, comp, toff, B, ldb, o, M, N, K, kb, ke, col0, vmax, pages);
 }
 
 __device__ __forceinline__ void add_slab(float (&s)[4], const uint2 v)
@@ -737,6 +845,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_pages_kernel(_Float16* __re
                                                                  int N,
                                                                  int split_k,
                                                                  int pages_per_unit,
+                                                                 int rows_per_unit,
                                                                  int col_groups,
                                                                  unsigned spmm_grid)
 {
@@ -747,6 +856,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_pages_kernel(_Float16* __re
     const unsigned units = gridDim.x / pages_per_unit;
     int            unit, sub;
     unit_of_workgroup(blockIdx.x, units, pages_per_unit, unit, sub);
+    if ((unit / col_groups) * rows_per_unit + sub / (pages_per_unit / rows_per_unit) >= M / kTileRows)
+        return;  // a row tile beyond the last one (the last unit of a launch may be short of row tiles)
     const uint4* first = ws + static_cast<size_t>(sub) * spmm_grid * (cols * 16) + t;
     float        s[8]  = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int k0 = 0; k0 < split_k; k0 += 8) {
@@ -771,9 +882,12 @@ __global__ __launch_bounds__(256) void splitk_reduce_pages_kernel(_Float16* __re
         hi[e] = static_cast<_Float16>(RELU && !(s[4 + e] > 0.f) ? 0.f : s[4 + e]);
     }
     // piece t = q*(4*cols) + g*cols + r16: rows 32q + 4g .. +3 and 16 further on, column r16 of the block
+    // a unit's pages: rows_per_unit row tiles, one after the other, each with the unit's 16-column blocks in order
     const int q = t / (4 * cols), g = (t / cols) & 3, r16 = t % cols;
-    const int n = ((unit % col_groups) * pages_per_unit + sub) * 16 + r16;
-    _Float16* o = c + static_cast<size_t>(n) * M + static_cast<size_t>(unit / col_groups) * kTileRows + q * 32 + g * 4;
+    const int blocks  = pages_per_unit / rows_per_unit;
+    const int n       = ((unit % col_groups) * blocks + sub % blocks) * 16 + r16;
+    const int rowtile = (unit / col_groups) * rows_per_unit + sub / blocks;
+    _Float16* o = c + static_cast<size_t>(n) * M + static_cast<size_t>(rowtile) * kTileRows + q * 32 + g * 4;
     *reinterpret_cast<half4*>(o)      = lo;
     *reinterpret_cast<half4*>(o + 16) = hi;
 }
@@ -806,18 +920,20 @@ __global__ __launch_bounds__(256) void take_rows_kernel(uint4* __restrict__ dst,
     dst[i] = src[static_cast<long>(j) * ld8 + r];
 }
 
-template<int NB, int DEPTH>
-int launch_spmm(hipStream_t stream, const void* comp, const int* offs, const void* b, void* out, int m, int n, int k, int split_k, int col_groups, int pages)
+template<int NB, int DEPTH, int W, int G>
+int launch_spmm(hipStream_t stream, const void* comp, const int* offs, const void* b, int ldb, void* out, int m, int n, int k, int split_k, int col_groups, int pages)
 {
-    const dim3 grid(static_cast<unsigned>(m / kTileRows) * col_groups * split_k, 1, 1);
-    hipLaunchKernelGGL((spmm_stream_kernel<NB, DEPTH>),
+    const unsigned row_units = (static_cast<unsigned>(m / kTileRows) + W - 1) / W;
+    const dim3     grid(row_units * col_groups * split_k, 1, 1);
+    hipLaunchKernelGGL((spmm_stream_kernel<NB, DEPTH, W, G>),
                        grid,
-                       dim3(kLanes),
+                       dim3(kLanes * W),
                        0,
                        stream,
                        static_cast<const uint4*>(comp),
                        offs,
                        static_cast<const _Float16*>(b),
+                       ldb,
                        static_cast<_Float16*>(out),
                        m,
                        n,
@@ -826,6 +942,22 @@ int launch_spmm(hipStream_t stream, const void* comp, const int* offs, const voi
                        col_groups,
                        pages);
     return static_cast<int>(hipGetLastError());
+}
+
+// Row tiles per workgroup of the launch for B of n columns and A of m rows: 8 for n = 64 when the number of row
+// tiles is a multiple of 8 (a CU's eight waves share each staged window of B; the slabs of whole workgroups then
+// fill Split_K*M*N halfs exactly, and the callers' workspaces hold no more), 1 otherwise.  Measured at
+// 36864 x 9216, 80 %: n = 64 62-64 us against 73.6 with one row tile per workgroup; n = 32 52.4 against 51.7
+// (the four fragment loads a tile costs there are no more than the meeting and the LDS reads that replace them),
+// and workgroups of four row tiles meeting at every tile gain nothing at n = 64 (72.9 us).
+// g_rows_override (a measuring aid) caps it at 1.
+std::atomic<int> g_rows_override{0};
+
+int rows_per_workgroup(int n, int m)
+{
+    if (n != 64 || g_rows_override.load(std::memory_order_relaxed) == 1)
+        return 1;
+    return (m / kTileRows) % 8 == 0 ? 8 : 1;
 }
 
 constexpr int      kMaxDevices = 64;
@@ -862,24 +994,36 @@ extern "C" int flashllm_hip_static_workspace(void** ptr)
 
 // pages != 0 (Split_K > 1 only): the slabs go to the workspace by workgroup, for flashllm_hip_launch_reduce_pages
 extern "C" int flashllm_hip_launch_spmm(
-    void* stream, const void* comp, const int* offs, const void* b, void* out, int m, int n, int k, int split_k, int pages)
+    void* stream, const void* comp, const int* offs, const void* b, int ldb, void* out, int m, int n, int k, int split_k, int pages)
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
     pages         = pages && split_k > 1;
     if (n <= 16)
-        return launch_spmm<1, 8>(s, comp, offs, b, out, m, n, k, split_k, 1, pages);
+        return launch_spmm<1, 8, 1, 1>(s, comp, offs, b, ldb, out, m, n, k, split_k, 1, pages);
     if (n == 32)
-        return launch_spmm<2, 8>(s, comp, offs, b, out, m, n, k, split_k, 1, pages);
-    return launch_spmm<4, 6>(s, comp, offs, b, out, m, n, k, split_k, n / 64, pages);
+        return launch_spmm<2, 8, 1, 1>(s, comp, offs, b, ldb, out, m, n, k, split_k, 1, pages);
+    if (rows_per_workgroup(n, m) == 8)
+        return launch_spmm<4, 8, 8, 2>(s, comp, offs, b, ldb, out, m, n, k, split_k, 1, pages);
+    return launch_spmm<4, 6, 1, 1>(s, comp, offs, b, ldb, out, m, n, k, split_k, n / 64, pages);
+}
+
+extern "C" void flashllm_hip_set_rows_per_workgroup(int rows)
+{
+    g_rows_override.store(rows, std::memory_order_relaxed);
+}
+
+extern "C" int flashllm_hip_rows_per_workgroup(int n, int m)
+{
+    return rows_per_workgroup(n, m);
 }
 
 extern "C" int flashllm_hip_launch_spmm_group(
-    void* stream, const void* comp, const int* offs, const void* b, void* out, int m, int n, int k, int split_k, int pages)
+    void* stream, const void* comp, const int* offs, const void* b, int ldb, void* out, int m, int n, int k, int split_k, int pages)
 {
     // 128 columns per workgroup (four waves x 32); requires n % 128 == 0
     const dim3 grid(static_cast<unsigned>(m / kTileRows) * (n / 128) * split_k, 1, 1);
     hipLaunchKernelGGL(spmm_group_kernel<2>, grid, dim3(kGroupThreads), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const uint4*>(comp), offs, static_cast<const _Float16*>(b), static_cast<_Float16*>(out),
+                       static_cast<const uint4*>(comp), offs, static_cast<const _Float16*>(b), ldb, static_cast<_Float16*>(out),
                        m, n, k, split_k, n / 128, pages && split_k > 1);
     return static_cast<int>(hipGetLastError());
 }
@@ -900,20 +1044,21 @@ extern "C" int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws,
 
 extern "C" int flashllm_hip_launch_reduce_pages(void* stream, void* c, const void* ws, int m, int n, int split_k, int relu)
 {
-    // the units of the SpMM launch for this N, 16*nb columns wide: one wave's columns in spmm_stream_kernel,
-    // a workgroup's 128 in spmm_group_kernel
+    // the units of the SpMM launch for this N: `rows` row tiles x 16*blocks columns (a wave's columns in
+    // spmm_stream_kernel, a workgroup's 128 in spmm_group_kernel)
     const bool     group      = n % 128 == 0;
-    const int      nb         = group ? 8 : (n <= 16 ? 1 : (n == 32 ? 2 : 4));
+    const int      rows       = group ? 1 : rows_per_workgroup(n, m);
+    const int      blocks     = group ? 8 : (n <= 16 ? 1 : (n == 32 ? 2 : 4));
     const int      col_groups = group ? n / 128 : (n <= 64 ? 1 : n / 64);
-    const unsigned units      = static_cast<unsigned>(m / kTileRows) * col_groups;
-    const dim3     grid(units * nb);
+    const unsigned units      = (static_cast<unsigned>(m / kTileRows) + rows - 1) / rows * col_groups;
+    const dim3     grid(units * blocks * rows);
     hipStream_t    s  = static_cast<hipStream_t>(stream);
     _Float16*      cp = static_cast<_Float16*>(c);
     const uint4*   wp = static_cast<const uint4*>(ws);
     if (relu)
-        hipLaunchKernelGGL(splitk_reduce_pages_kernel<true>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, nb, col_groups, units * split_k);
+        hipLaunchKernelGGL(splitk_reduce_pages_kernel<true>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, blocks * rows, rows, col_groups, units * split_k);
     else
-        hipLaunchKernelGGL(splitk_reduce_pages_kernel<false>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, nb, col_groups, units * split_k);
+        hipLaunchKernelGGL(splitk_reduce_pages_kernel<false>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, blocks * rows, rows, col_groups, units * split_k);
     return static_cast<int>(hipGetLastError());
 }
 

@@ -21,11 +21,13 @@ int flashllm_hip_static_workspace(void** ptr);
 // pages == 0: slab s is M*N halfs at s*M*N, laid out like C (for flashllm_hip_launch_reduce);
 // pages != 0: each workgroup's 128 x 16 blocks of partial sums as 4 KB pages in workgroup order
 // (for flashllm_hip_launch_reduce_pages; needs out 16-byte aligned).
+// ldb: halfs between consecutive columns of B (>= K, a multiple of 8; K for a dense column-major B).
 // Requires M % 128 == 0, K % 64 == 0, N in {8,16,32,64} or N % 64 == 0.
 int flashllm_hip_launch_spmm(void*       stream,
                              const void* compressed_a,
                              const int*  tile_offsets,
                              const void* b,
+                             int         ldb,
                              void*       out,
                              int         m,
                              int         n,
@@ -33,11 +35,19 @@ int flashllm_hip_launch_spmm(void*       stream,
                              int         split_k,
                              int         pages);
 
+// Row tiles per workgroup of flashllm_hip_launch_spmm for n columns and m rows: 8 for n = 64 when m / 128 is a
+// multiple of 8, otherwise 1.  flashllm_hip_set_rows_per_workgroup(1) is a measuring aid that forces 1 (anything
+// else: the default), process-wide; the launch of the partial products and the reduction of its pages must see
+// the same value.
+void flashllm_hip_set_rows_per_workgroup(int rows);
+int  flashllm_hip_rows_per_workgroup(int n, int m);
+
 // The same product for wide B (n % 128 == 0) by workgroups of four waves that share each scattered tile.
 int flashllm_hip_launch_spmm_group(void*       stream,
                                    const void* compressed_a,
                                    const int*  tile_offsets,
                                    const void* b,
+                                   int         ldb,
                                    void*       out,
                                    int         m,
                                    int         n,

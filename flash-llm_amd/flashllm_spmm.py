@@ -288,8 +288,10 @@ class DecoderLayer:
             need = max(need, s * w.m * tokens)
         return need
 
-    def forward(self, x, tokens, buffers=None, workspace=None, stream=None):
-        """x: fp16 device tensor, column-major hidden x tokens.  Returns (y, buffers)."""
+    def forward(self, x, tokens, buffers=None, workspace=None, stream=None, copy_attn_in=False):
+        """x: fp16 device tensor, column-major hidden x tokens.  Returns (y, buffers); buffers = [qkv_out, attn_in,
+        attn_out, ffn_mid, y].  attn_in is only written with copy_attn_in=True: the attention-output linear reads
+        the first hidden rows of qkv_out in place."""
         import torch
 
         qkv, o, f1, f2 = self.weights
@@ -298,8 +300,10 @@ class DecoderLayer:
             buffers = [torch.empty(n * tokens, dtype=torch.float16, device=dev) for n in (qkv.m, o.k, o.m, f1.m, f2.m)]
         if workspace is None:
             workspace = torch.empty(self.workspace_halfs(tokens), dtype=torch.float16, device=dev)
-        rc = lib().flashllm_decoder_layer_linears(_stream(stream), ctypes.byref(self.struct), _ptr(x), *[_ptr(b) for b in buffers],
-                                                  tokens, _ptr(workspace))
+        ptrs = [_ptr(b) for b in buffers]
+        if not copy_attn_in:
+            ptrs[1] = None
+        rc = lib().flashllm_decoder_layer_linears(_stream(stream), ctypes.byref(self.struct), _ptr(x), *ptrs, tokens, _ptr(workspace))
         if rc:
             raise HipError(rc)
         return buffers[4], buffers

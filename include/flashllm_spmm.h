@@ -208,8 +208,9 @@ typedef struct {
  *     ffn_mid  = relu(W1 * attn_out)
  *     y        = W2   * ffn_mid
  * Like the reference's call sites, Split_K falls back to 1 when tokens > 128 (FFN, ft.patch:523)
- * or tokens > 64 (attention, ft.patch:1454).  attn_in (hidden x tokens) receives the first hidden
- * rows of every column of qkv_out (a strided copy kernel), because B must be dense column-major.
+ * or tokens > 64 (attention, ft.patch:1454).  The attention-output linear reads the first hidden rows
+ * of every column of qkv_out in place (B with its columns qkv.m halfs apart).  attn_in may be NULL; when
+ * it is not, it also receives those rows as a dense hidden x tokens matrix (a strided copy kernel).
  * Buffers: qkv_out qkv.m*tokens, attn_in / attn_out attn_out.k*tokens / attn_out.m*tokens,
  * ffn_mid ffn1.m*tokens, y ffn2.m*tokens halfs; workspace for the largest Split_K*M*tokens.
  * Returns a hipError_t as int (hipErrorInvalidValue when the shapes do not chain).

@@ -128,8 +128,7 @@ def test_decoder_layers_hidden9216_eight_layers(product, oracle, torch_gpu):
         qkv = qkv.reshape(tokens, 3 * hidden)
         ref, _ = oracle.gemm_f32(dense[0], x_h, tokens)
         assert_close(qkv, ref, f"layer {layer} qkv")
-        attn_in = attn_in.reshape(tokens, hidden)
-        assert np.array_equal(attn_in.view(np.uint16), np.ascontiguousarray(qkv[:, :hidden]).view(np.uint16))
+        attn_in = np.ascontiguousarray(qkv[:, :hidden])   # read in place by the attention-output linear
         ref, _ = oracle.gemm_f32(dense[1], attn_in, tokens)
         attn_out = attn_out.reshape(tokens, hidden)
         assert_close(attn_out, ref, f"layer {layer} attention output")

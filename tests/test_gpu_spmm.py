@@ -233,8 +233,9 @@ def test_split_k_reduction_of_slabs_by_workgroup_bit_exact(product, oracle, torc
     torch = torch_gpu
     rng = np.random.default_rng(21)
     # 8 and 16 row tiles fill whole XCD rounds, 1 / 3 / 11 leave units beyond a multiple of eight
+    # N = 32 / 64: workgroups of 8 row tiles (2048 and 1024 rows), of 4 (512 and 1536), of 1 (256 and 1408)
     for m, n, s in [(128, 8, 2), (1024, 16, 7), (256, 64, 32), (384, 8, 5), (2048, 32, 9), (1024, 128, 3), (256, 256, 11),
-                    (1408, 16, 4), (1408, 64, 3)]:
+                    (1408, 16, 4), (1408, 64, 3), (1024, 64, 5), (512, 32, 3), (1536, 64, 2), (3072, 32, 4)]:
         say(f"reduction of pages m={m} n={n} s={s}")
         ws_h = (rng.standard_normal((s, n * m)) * 3).astype(np.float16)
         ws = torch.from_numpy(slab_pages(ws_h, m, n)).cuda()
@@ -257,7 +258,8 @@ def test_workgroups_go_round_robin_over_the_xcds(product, torch_gpu):
     assert distinct in (1, 2, 4, 8)  # whole GPU, or one of its partition modes
 
 
-@pytest.mark.parametrize("m,n,k,s", [(512, 16, 1024, 4), (1152, 8, 512, 3), (1280, 64, 512, 2), (384, 128, 768, 3)])
+@pytest.mark.parametrize("m,n,k,s", [(512, 16, 1024, 4), (1152, 8, 512, 3), (1280, 64, 512, 2), (384, 128, 768, 3),
+                                     (1024, 64, 1024, 3), (2048, 32, 1536, 5), (512, 32, 640, 2), (1536, 64, 448, 4)])
 def test_partials_then_reduce_equals_api(product, oracle, torch_gpu, m, n, k, s):
     """Both slab orders hold the same partial sums (each the oracle's product over its K slice), and the
     two halves called separately give the API's C in either order."""
@@ -387,9 +389,19 @@ def test_decoder_layer_chain(product, oracle, torch_gpu, tokens):
     layer = product.DecoderLayer(*weights)
     x_h = synth.dense_b(hidden, tokens, 30, dist="normal")
     x = torch.from_numpy(x_h).cuda()
-    y, bufs = layer.forward(x, tokens)
+    # with the optional contiguous copy of the attention-output linear's input, then without (the linear reads
+    # qkv_out in place either way): every buffer must come out the same
+    y, bufs = layer.forward(x, tokens, copy_attn_in=True)
     torch.cuda.synchronize()
-    qkv, attn_in, attn_out, ffn_mid, y = [b.cpu().numpy() for b in bufs]
+    first = [b.clone() for b in bufs]
+    for b in bufs:
+        b.fill_(float("nan"))
+    y, bufs = layer.forward(x, tokens, buffers=bufs)
+    torch.cuda.synchronize()
+    assert torch.isnan(bufs[1]).all()   # not written without copy_attn_in
+    for i in (0, 2, 3, 4):
+        assert torch.equal(bufs[i].view(torch.int16), first[i].view(torch.int16)), i
+    qkv, attn_in, attn_out, ffn_mid, y = [b.cpu().numpy() for b in first]
     qkv = qkv.reshape(tokens, 3 * hidden)
     ref, _ = oracle.gemm_f32(dense[0], x_h, tokens)
     assert_close(qkv, ref, "qkv")

@@ -102,7 +102,7 @@ def test_slab_page_layout_helper_is_a_bijection_with_known_corners():
     a permutation of the S*N*M halfs, and a few entries placed by hand from the layout's description."""
     from gpu_util import slab_pages, slabs_from_pages
 
-    for m, n, s in [(128, 8, 2), (1024, 16, 7), (1408, 64, 3), (256, 256, 11), (384, 128, 3)]:
+    for m, n, s in [(128, 8, 2), (1024, 16, 7), (1408, 64, 3), (256, 256, 11), (384, 128, 3), (1024, 64, 3), (2048, 32, 5), (512, 32, 2), (1536, 64, 4)]:
         x = np.arange(s * n * m, dtype=np.int64).reshape(s, n, m)
         p = slab_pages(x, m, n)
         assert np.array_equal(np.sort(p), np.arange(s * n * m))
@@ -119,3 +119,15 @@ def test_slab_page_layout_helper_is_a_bijection_with_known_corners():
     assert p[2048 * 1] == x[0, 0, 128]                       # workgroup 1 = unit 1 (row tile 1), slice 0
     assert p[2048 * 8] == x[1, 0, 0]                         # workgroup 8 = unit 0, slice 1
     assert p[2048 * (6 * 8 + 5) + 8 * (2 * 64 + 3 * 16 + 9) + 6] == x[6, 9, 5 * 128 + 64 + 16 + 12 + 2]
+    # M = 2048 (16 row tiles), N = 64, S = 3: workgroups of 8 row tiles, so 2 units (fewer than 8: workgroup =
+    # unit*S + slice) and a launch of G = 6 workgroups; a unit's 32 pages are (row tile r, block b) -> sub = 4r + b
+    # at page sub*G + workgroup
+    m, n, s = 2048, 64, 3
+    x = np.arange(s * n * m, dtype=np.int64).reshape(s, n, m)
+    p = slab_pages(x, m, n)
+    assert p[0] == x[0, 0, 0]
+    assert p[2048 * (1 * 6 + 0)] == x[0, 16, 0]              # sub 1: row tile 0, columns 16..31
+    assert p[2048 * (4 * 6 + 0)] == x[0, 0, 128]             # sub 4: row tile 1, columns 0..15
+    assert p[2048 * (0 * 6 + 1)] == x[1, 0, 0]               # workgroup 1 = unit 0, slice 1
+    assert p[2048 * (0 * 6 + 3)] == x[0, 0, 8 * 128]         # workgroup 3 = unit 1 (row tiles 8..15), slice 0
+    assert p[2048 * (31 * 6 + 5) + 8 * 17 + 1] == x[2, 48 + 1, 15 * 128 + 4 + 1]   # last page: piece 17 = g 1, column 1

@@ -1055,10 +1055,12 @@ extern "C" int flashllm_hip_launch_reduce_pages(void* stream, void* c, const voi
     hipStream_t    s  = static_cast<hipStream_t>(stream);
     _Float16*      cp = static_cast<_Float16*>(c);
     const uint4*   wp = static_cast<const uint4*>(ws);
+    const int pages_per_unit = blocks * rows;
+    const unsigned spmm_grid = units * split_k;
     if (relu)
-        hipLaunchKernelGGL(splitk_reduce_pages_kernel<true>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, blocks * rows, rows, col_groups, units * split_k);
+        hipLaunchKernelGGL(splitk_reduce_pages_kernel<true>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, pages_per_unit, rows, col_groups, spmm_grid);
     else
-        hipLaunchKernelGGL(splitk_reduce_pages_kernel<false>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, blocks * rows, rows, col_groups, units * split_k);
+        hipLaunchKernelGGL(splitk_reduce_pages_kernel<false>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, pages_per_unit, rows, col_groups, spmm_grid);
     return static_cast<int>(hipGetLastError());
 }
 

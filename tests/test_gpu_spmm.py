@@ -90,6 +90,77 @@ def test_ragged_tiles_and_empty_slices(product, oracle, torch_gpu):
         assert_close(c, ref, f"ragged split_k={split_k}")
 
 
+# --- N = 64 with a multiple of eight row tiles: workgroups of eight waves sharing B through LDS ------------
+def eight_row_tile_matrix(seed):
+    """1024 x 640: eight row tiles (one workgroup of eight waves per K slice) whose waves meet very different
+    slices: a tile row without any nonzero, one with a single nonzero, empty tiles at the start, in the middle
+    and at the end of a row, a full tile, a row that is dense throughout."""
+    m, k = 1024, 640
+    a = synth.sparse_matrix(m, k, 0.8, seed)
+    a[0:128, 0:64] = 0            # tile row 0: first tile empty
+    a[0:128, 256:384] = 0         #             two empty tiles in the middle
+    a[128:256, :] = 0             # tile row 1: nothing at all (its wave only attends the meetings)
+    a[256:384, :] = 0
+    a[300, 200] = -2.5            # tile row 2: one nonzero, one vector with three paddings
+    a[384:512, 576:640] = 0       # tile row 3: last tile empty
+    a[512:640, 448:512] = synth.sparse_matrix(128, 64, 0.0, seed + 1)   # tile row 4: a full tile
+    a[640:768, :] = synth.sparse_matrix(128, k, 0.0, seed + 2)          # tile row 5: dense throughout
+    a[768:896, 64:] = 0           # tile row 6: only its first tile holds anything
+    return a
+
+
+def test_eight_wave_workgroups_ragged_rows_and_empty_slices(product, oracle, torch_gpu):
+    say("N=64, eight row tiles per workgroup: ragged rows")
+    assert product.lib().flashllm_hip_rows_per_workgroup(64, 1024) == 8
+    a = eight_row_tile_matrix(60)
+    b = synth.dense_b(640, 64, 61)
+    for split_k in (1, 2, 3, 5, 10, 16):   # windows of two k tiles: slices of 10, 5, 4 (and 2), 2, 1 and 0 k tiles
+        c, _, _ = run_spmm(product, a, b, 64, split_k)
+        _, ref = oracle.spmm_model(a, b, 64, split_k)
+        assert not c[:, 128:256].any()
+        assert_close(c, ref, f"eight-wave ragged split_k={split_k}")
+
+
+@pytest.mark.parametrize("sparsity", [0.0, 0.5, 0.8, 0.95, 0.999, 1.0])
+def test_eight_wave_workgroups_any_density(product, oracle, torch_gpu, sparsity):
+    say(f"N=64, eight row tiles per workgroup: sparsity={sparsity}")
+    a = synth.sparse_matrix(1024, 768, sparsity, 62)
+    b = synth.dense_b(768, 64, 63)
+    for split_k in (1, 3, 4):
+        c, _, _ = run_spmm(product, a, b, 64, split_k)
+        _, ref = oracle.spmm_model(a, b, 64, split_k)
+        if sparsity == 1.0:
+            assert not c.any()
+        else:
+            assert_close(c, ref, f"eight-wave sparsity={sparsity} split_k={split_k}")
+
+
+def test_eight_wave_workgroups_match_single_wave_workgroups_bit_for_bit(product, torch_gpu):
+    """Where B comes from does not change a sum: with the library told to use one row tile per workgroup (every
+    wave fetching its own B fragments) C and the slabs must be the same bits."""
+    torch = torch_gpu
+    say("N=64: eight-wave against one-wave workgroups")
+    L = product.lib()
+    b_h = synth.dense_b(640, 64, 65, dist="normal")
+    for a in (eight_row_tile_matrix(64), synth.sparse_matrix(2048, 640, 0.8, 66, dist="normal", sigma=0.05)):
+        m, k = a.shape
+        w = product.SparseWeight(a)
+        b = torch.from_numpy(b_h).cuda()
+        for split_k in (1, 3, 7):
+            got = []
+            for cap in (0, 1):
+                L.flashllm_hip_set_rows_per_workgroup(cap)
+                try:
+                    c = torch.full((64 * m,), float("nan"), dtype=torch.float16, device="cuda")
+                    ws = torch.full((split_k * 64 * m,), float("nan"), dtype=torch.float16, device="cuda")
+                    product.spmm_partials(w.comp, w.offs, b, c, m, 64, k, ws, split_k)   # plain slabs: the same layout either way
+                    torch.cuda.synchronize()
+                    got.append((c if split_k == 1 else ws).cpu().numpy().view(np.uint16).copy())
+                finally:
+                    L.flashllm_hip_set_rows_per_workgroup(0)
+            assert np.array_equal(got[0], got[1]), f"m={m} split_k={split_k}"
+
+
 # --- the four-wave kernel for wide B (N a multiple of 128) -------------------------------------------
 @pytest.mark.parametrize("n", [128, 384])
 @pytest.mark.parametrize("sparsity", [0.0, 0.5, 0.72, 0.8, 0.95, 0.999, 1.0])
@@ -154,7 +225,7 @@ def test_empty_matrix_with_a_four_byte_allocation(product, torch_gpu, n):
     (kernel_benchmark/spmm_test.cu:258-260).  No kernel may count on more."""
     torch = torch_gpu
     say(f"empty matrix, one-element Compressed_A, n={n}")
-    m, k = 512, 1024
+    m, k = 1024, 1024
     a = np.zeros((m, k), dtype=np.float16)
     items, offsets = product.init_sparse_matrix_a(a)
     assert items.size == 0 and not offsets.any()
@@ -375,14 +446,14 @@ def test_nonuniform_rows(product, oracle, torch_gpu):
 
 
 # --- config 5 flavour: the four linears of a decoder layer, chained --------------------------------
-@pytest.mark.parametrize("tokens", [16, 256])
-def test_decoder_layer_chain(product, oracle, torch_gpu, tokens):
+@pytest.mark.parametrize("tokens,hidden", [(16, 512), (256, 512), (64, 1024)])
+def test_decoder_layer_chain(product, oracle, torch_gpu, tokens, hidden):
     """QKV -> (first hidden rows) -> attention output -> FFN1 -> ReLU -> FFN2 on one stream with one
     workspace; every stage is checked against an fp32 product of the previous stage's fp16 output.
-    tokens = 256 exercises the reference's fallback to Split_K = 1 (ft.patch:523, :1454)."""
+    tokens = 256 exercises the reference's fallback to Split_K = 1 (ft.patch:523, :1454); 64 tokens at hidden 1024 take
+    the eight-wave workgroups of N = 64, the attention-output linear with B read in place at leading dimension 3072."""
     torch = torch_gpu
-    say(f"decoder layer chain tokens={tokens}")
-    hidden = 512
+    say(f"decoder layer chain tokens={tokens} hidden={hidden}")
     shapes = [(3 * hidden, hidden), (hidden, hidden), (4 * hidden, hidden), (hidden, 4 * hidden)]
     dense = [synth.sparse_matrix(m, k, 0.8, 20 + i, dist="normal", sigma=0.05) for i, (m, k) in enumerate(shapes)]
     weights = [product.SparseWeight(a) for a in dense]

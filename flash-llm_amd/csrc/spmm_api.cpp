@@ -244,20 +244,21 @@ int flashllm_splitk_heuristic(int m, int n, int k)
     const int    col_groups = n <= 64 ? 1 : n / 64;
     const long   units      = static_cast<long>(m / 128) * col_groups;
     const long   slots      = 256L * 8;
-    // N = 64 with eight row tiles per workgroup (a workgroup fills a CU): the same form fitted to the same twelve
-    // shapes again, mean 0.5 %, at most 5.7 % above the best.  Crowding costs less there (the waves of a CU no
-    // longer fetch B eight times), so the pick is mostly the largest Split_K whose workgroups fit the 256 CUs.
-    const bool   by_eight   = flashllm_hip_rows_per_workgroup(n, m) == 8;
-    const double fixed      = by_eight ? 4.0 : 2.0;
-    const double crowding   = by_eight ? 0.5 : 1.0;
-    const double per_slab   = by_eight ? 1.0 + 0.125 * (n / 16.0) * (m / 36864.0) : 0.5 + 0.5 * (n / 16.0) * (m / 36864.0);
     int          best       = 1;
     double       best_cost  = 1e30;
     for (int s = 1; s <= 32 && s <= kt; s++) {  // workspace sizes in existing callers assume at most 32 slabs
         if (s > 1 && units * s > slots)
             break;
-        const int    longest = (kt - 1) / s + 1;
-        const double cost    = longest * (fixed + crowding * units * s / 256.0) + (s > 1 ? s * per_slab : 0.0);
+        // N = 64 with eight row tiles per workgroup (what the launch does for this Split_K when its workgroups
+        // fill between three quarters and all of the CUs): the same form fitted to the same twelve shapes again,
+        // mean 0.5 %, at most 5.7 % above the best.  Crowding costs less there (the waves of a CU no longer fetch
+        // B eight times), so the pick is mostly the largest Split_K whose workgroups fit the 256 CUs.
+        const bool   by_eight = flashllm_hip_rows_per_workgroup(n, m, s) == 8;
+        const double fixed    = by_eight ? 4.0 : 2.0;
+        const double crowding = by_eight ? 0.5 : 1.0;
+        const double per_slab = by_eight ? 1.0 + 0.125 * (n / 16.0) * (m / 36864.0) : 0.5 + 0.5 * (n / 16.0) * (m / 36864.0);
+        const int    longest  = (kt - 1) / s + 1;
+        const double cost     = longest * (fixed + crowding * units * s / 256.0) + (s > 1 ? s * per_slab : 0.0);
         if (cost < best_cost) {
             best_cost = cost;
             best      = s;

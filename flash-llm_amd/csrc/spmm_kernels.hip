@@ -944,20 +944,28 @@ int launch_spmm(hipStream_t stream, const void* comp, const int* offs, const voi
     return static_cast<int>(hipGetLastError());
 }
 
-// Row tiles per workgroup of the launch for B of n columns and A of m rows: 8 for n = 64 when the number of row
-// tiles is a multiple of 8 (a CU's eight waves share each staged window of B; the slabs of whole workgroups then
-// fill Split_K*M*N halfs exactly, and the callers' workspaces hold no more), 1 otherwise.  Measured at
-// 36864 x 9216, 80 %: n = 64 62-64 us against 73.6 with one row tile per workgroup; n = 32 52.4 against 51.7
-// (the four fragment loads a tile costs there are no more than the meeting and the LDS reads that replace them),
-// and workgroups of four row tiles meeting at every tile gain nothing at n = 64 (72.9 us).
-// g_rows_override (a measuring aid) caps it at 1.
+// Row tiles per workgroup of the launch for B of n columns, A of m rows and split_k slices: 8 (a CU's eight waves
+// share each staged window of B) for n = 64 when the row tiles come in whole groups of eight (the slabs of whole
+// workgroups then fill Split_K*M*N halfs exactly, and the callers' workspaces hold no more) and the launch's
+// workgroups, each of which fills a CU, number between 192 and 256: one round on at least three quarters of the
+// 256 CUs.  Otherwise 1: fewer, larger workgroups would leave CUs idle (7168 x 7168 at its best Split_K: 23.8 us
+// with one row tile per workgroup, 29.6 us with eight), more would run in two rounds.
+// Measured at 36864 x 9216, 80 %: n = 64 62-64 us against 73.6 with one row tile per workgroup; n = 32 52.4
+// against 51.7 (the four fragment loads a tile costs there are no more than the meeting and the LDS reads that
+// replace them), and workgroups of four row tiles meeting at every tile gain nothing at n = 64 (72.9 us).
+// g_rows_override (a measuring and testing aid): 1 forces 1, 8 forces 8 wherever the row tiles allow it.
 std::atomic<int> g_rows_override{0};
 
-int rows_per_workgroup(int n, int m)
+int rows_per_workgroup(int n, int m, int split_k)
 {
-    if (n != 64 || g_rows_override.load(std::memory_order_relaxed) == 1)
+    const int forced = g_rows_override.load(std::memory_order_relaxed);
+    const int tiles  = m / kTileRows;
+    if (n != 64 || forced == 1 || tiles % 8)
         return 1;
-    return (m / kTileRows) % 8 == 0 ? 8 : 1;
+    if (forced == 8)
+        return 8;
+    const long workgroups = static_cast<long>(tiles / 8) * split_k;
+    return workgroups >= 192 && workgroups <= 256 ? 8 : 1;
 }
 
 constexpr int      kMaxDevices = 64;
@@ -1002,7 +1010,7 @@ extern "C" int flashllm_hip_launch_spmm(
         return launch_spmm<1, 8, 1, 1>(s, comp, offs, b, ldb, out, m, n, k, split_k, 1, pages);
     if (n == 32)
         return launch_spmm<2, 8, 1, 1>(s, comp, offs, b, ldb, out, m, n, k, split_k, 1, pages);
-    if (rows_per_workgroup(n, m) == 8)
+    if (rows_per_workgroup(n, m, split_k) == 8)
         return launch_spmm<4, 8, 8, 2>(s, comp, offs, b, ldb, out, m, n, k, split_k, 1, pages);
     return launch_spmm<4, 6, 1, 1>(s, comp, offs, b, ldb, out, m, n, k, split_k, n / 64, pages);
 }
@@ -1012,9 +1020,9 @@ extern "C" void flashllm_hip_set_rows_per_workgroup(int rows)
     g_rows_override.store(rows, std::memory_order_relaxed);
 }
 
-extern "C" int flashllm_hip_rows_per_workgroup(int n, int m)
+extern "C" int flashllm_hip_rows_per_workgroup(int n, int m, int split_k)
 {
-    return rows_per_workgroup(n, m);
+    return rows_per_workgroup(n, m, split_k);
 }
 
 extern "C" int flashllm_hip_launch_spmm_group(
@@ -1047,7 +1055,7 @@ extern "C" int flashllm_hip_launch_reduce_pages(void* stream, void* c, const voi
     // the units of the SpMM launch for this N: `rows` row tiles x 16*blocks columns (a wave's columns in
     // spmm_stream_kernel, a workgroup's 128 in spmm_group_kernel)
     const bool     group      = n % 128 == 0;
-    const int      rows       = group ? 1 : rows_per_workgroup(n, m);
+    const int      rows       = group ? 1 : rows_per_workgroup(n, m, split_k);
     const int      blocks     = group ? 8 : (n <= 16 ? 1 : (n == 32 ? 2 : 4));
     const int      col_groups = group ? n / 128 : (n <= 64 ? 1 : n / 64);
     const unsigned units      = (static_cast<unsigned>(m / kTileRows) + rows - 1) / rows * col_groups;

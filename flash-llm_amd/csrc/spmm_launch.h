@@ -35,12 +35,13 @@ int flashllm_hip_launch_spmm(void*       stream,
                              int         split_k,
                              int         pages);
 
-// Row tiles per workgroup of flashllm_hip_launch_spmm for n columns and m rows: 8 for n = 64 when m / 128 is a
-// multiple of 8, otherwise 1.  flashllm_hip_set_rows_per_workgroup(1) is a measuring aid that forces 1 (anything
-// else: the default), process-wide; the launch of the partial products and the reduction of its pages must see
-// the same value.
+// Row tiles per workgroup of flashllm_hip_launch_spmm for n columns, m rows and split_k slices: 8 for n = 64
+// when m / 128 is a multiple of 8 and (m / 1024) * split_k lies in 192 .. 256, otherwise 1.
+// flashllm_hip_set_rows_per_workgroup is a measuring and testing aid, process-wide: 1 forces 1, 8 forces 8
+// wherever m / 128 is a multiple of 8, anything else restores the rule.  The launch of the partial products and
+// the reduction of its pages must see the same setting.
 void flashllm_hip_set_rows_per_workgroup(int rows);
-int  flashllm_hip_rows_per_workgroup(int n, int m);
+int  flashllm_hip_rows_per_workgroup(int n, int m, int split_k);
 
 // The same product for wide B (n % 128 == 0) by workgroups of four waves that share each scattered tile.
 int flashllm_hip_launch_spmm_group(void*       stream,

@@ -43,8 +43,8 @@ def slab_pages(slabs, m, n, rows=None):
     """Plain slabs (S, N, M) -> the same numbers in the by-workgroup order of the library (flat, S*N*M).
 
     Written from the layout's description, not from the kernels: a launch has units = (M/128) / rows x column
-    groups; a unit is `rows` consecutive row tiles (8 for N = 64 when M/128 is a multiple of 8: workgroups of eight
-    waves with a row tile each; otherwise 1) by 16*nb columns (nb = 1 / 2 / 4 for N <= 16 / 32 / 64, 8 and 128-column
+    groups; a unit is `rows` consecutive row tiles (8 for N = 64 when M/128 is a multiple of 8 and the launch has
+    192 .. 256 workgroups of eight waves with a row tile each, (M/1024)*S; otherwise 1; `rows` given: that) by 16*nb columns (nb = 1 / 2 / 4 for N <= 16 / 32 / 64, 8 and 128-column
     groups for wide B); workgroup w = ((unit % per_xcd)*S + slice)*8 + unit // per_xcd with per_xcd = units // 8
     (units past a multiple of 8: w = unit*S + slice); the unit's pages are numbered row tile by row tile, the
     16-column blocks of a row tile in order (sub = row*nb + block), page sub*G + w; and inside a page the
@@ -55,7 +55,7 @@ def slab_pages(slabs, m, n, rows=None):
     wide = n % 128 == 0
     nb = 8 if wide else (1 if n <= 16 else (2 if n == 32 else 4))
     if rows is None:
-        rows = 8 if n == 64 and (m // 128) % 8 == 0 else 1
+        rows = 8 if n == 64 and (m // 128) % 8 == 0 and 192 <= (m // 1024) * s <= 256 else 1
     assert (m // 128) % rows == 0
     col_groups = n // 128 if wide else 1
     cols = 8 if n < 16 else 16

@@ -21,6 +21,15 @@ def say(*a):
     sys.stdout.flush()
 
 
+@pytest.fixture
+def eight_row_tiles(product):
+    """Makes the N = 64 launches of a test use workgroups of eight row tiles at any size (by itself the library
+    takes them only when such workgroups fill most of the GPU); restored afterwards."""
+    product.lib().flashllm_hip_set_rows_per_workgroup(8)
+    yield
+    product.lib().flashllm_hip_set_rows_per_workgroup(0)
+
+
 @pytest.fixture(scope="module")
 def torch_gpu():
     import torch
@@ -109,9 +118,9 @@ def eight_row_tile_matrix(seed):
     return a
 
 
-def test_eight_wave_workgroups_ragged_rows_and_empty_slices(product, oracle, torch_gpu):
+def test_eight_wave_workgroups_ragged_rows_and_empty_slices(product, oracle, torch_gpu, eight_row_tiles):
     say("N=64, eight row tiles per workgroup: ragged rows")
-    assert product.lib().flashllm_hip_rows_per_workgroup(64, 1024) == 8
+    assert product.lib().flashllm_hip_rows_per_workgroup(64, 1024, 3) == 8
     a = eight_row_tile_matrix(60)
     b = synth.dense_b(640, 64, 61)
     for split_k in (1, 2, 3, 5, 10, 16):   # windows of two k tiles: slices of 10, 5, 4 (and 2), 2, 1 and 0 k tiles
@@ -122,7 +131,7 @@ def test_eight_wave_workgroups_ragged_rows_and_empty_slices(product, oracle, tor
 
 
 @pytest.mark.parametrize("sparsity", [0.0, 0.5, 0.8, 0.95, 0.999, 1.0])
-def test_eight_wave_workgroups_any_density(product, oracle, torch_gpu, sparsity):
+def test_eight_wave_workgroups_any_density(product, oracle, torch_gpu, sparsity, eight_row_tiles):
     say(f"N=64, eight row tiles per workgroup: sparsity={sparsity}")
     a = synth.sparse_matrix(1024, 768, sparsity, 62)
     b = synth.dense_b(768, 64, 63)
@@ -148,7 +157,7 @@ def test_eight_wave_workgroups_match_single_wave_workgroups_bit_for_bit(product,
         b = torch.from_numpy(b_h).cuda()
         for split_k in (1, 3, 7):
             got = []
-            for cap in (0, 1):
+            for cap in (8, 1):
                 L.flashllm_hip_set_rows_per_workgroup(cap)
                 try:
                     c = torch.full((64 * m,), float("nan"), dtype=torch.float16, device="cuda")
@@ -304,12 +313,28 @@ def test_split_k_reduction_of_slabs_by_workgroup_bit_exact(product, oracle, torc
     torch = torch_gpu
     rng = np.random.default_rng(21)
     # 8 and 16 row tiles fill whole XCD rounds, 1 / 3 / 11 leave units beyond a multiple of eight
-    # N = 32 / 64: workgroups of 8 row tiles (2048 and 1024 rows), of 4 (512 and 1536), of 1 (256 and 1408)
     for m, n, s in [(128, 8, 2), (1024, 16, 7), (256, 64, 32), (384, 8, 5), (2048, 32, 9), (1024, 128, 3), (256, 256, 11),
                     (1408, 16, 4), (1408, 64, 3), (1024, 64, 5), (512, 32, 3), (1536, 64, 2), (3072, 32, 4)]:
         say(f"reduction of pages m={m} n={n} s={s}")
         ws_h = (rng.standard_normal((s, n * m)) * 3).astype(np.float16)
         ws = torch.from_numpy(slab_pages(ws_h, m, n)).cuda()
+        c = torch.full((n * m,), float("nan"), dtype=torch.float16, device="cuda")
+        product.splitk_reduce(c, ws, m, n, s, slab_order=product.SLABS_BY_WORKGROUP)
+        torch.cuda.synchronize()
+        want = oracle.splitk_reduce(ws_h, n * m, s)
+        assert np.array_equal(c.cpu().numpy().view(np.uint16), want.view(np.uint16))
+
+
+def test_split_k_reduction_of_pages_of_eight_row_tile_workgroups_bit_exact(product, oracle, torch_gpu, eight_row_tiles):
+    """The same for the pages N = 64 launches leave when their workgroups take eight row tiles each: one unit
+    (1024 rows), three (units beyond whole XCD rounds), eight and nine."""
+    torch = torch_gpu
+    rng = np.random.default_rng(22)
+    for m, s in [(1024, 5), (3072, 2), (8192, 3), (9216, 28)]:
+        say(f"reduction of pages, eight row tiles per workgroup, m={m} s={s}")
+        n = 64
+        ws_h = (rng.standard_normal((s, n * m)) * 3).astype(np.float16)
+        ws = torch.from_numpy(slab_pages(ws_h, m, n, rows=8)).cuda()
         c = torch.full((n * m,), float("nan"), dtype=torch.float16, device="cuda")
         product.splitk_reduce(c, ws, m, n, s, slab_order=product.SLABS_BY_WORKGROUP)
         torch.cuda.synchronize()
@@ -330,8 +355,17 @@ def test_workgroups_go_round_robin_over_the_xcds(product, torch_gpu):
 
 
 @pytest.mark.parametrize("m,n,k,s", [(512, 16, 1024, 4), (1152, 8, 512, 3), (1280, 64, 512, 2), (384, 128, 768, 3),
-                                     (1024, 64, 1024, 3), (2048, 32, 1536, 5), (512, 32, 640, 2), (1536, 64, 448, 4)])
+                                     (2048, 32, 1536, 5), (1536, 64, 448, 4)])
 def test_partials_then_reduce_equals_api(product, oracle, torch_gpu, m, n, k, s):
+    check_partials_then_reduce(product, oracle, torch_gpu, m, n, k, s, None)
+
+
+@pytest.mark.parametrize("m,n,k,s", [(1024, 64, 1024, 3), (2048, 64, 1280, 5)])
+def test_partials_then_reduce_equals_api_eight_row_tile_workgroups(product, oracle, torch_gpu, eight_row_tiles, m, n, k, s):
+    check_partials_then_reduce(product, oracle, torch_gpu, m, n, k, s, 8)
+
+
+def check_partials_then_reduce(product, oracle, torch_gpu, m, n, k, s, rows):
     """Both slab orders hold the same partial sums (each the oracle's product over its K slice), and the
     two halves called separately give the API's C in either order."""
     torch = torch_gpu
@@ -346,7 +380,7 @@ def test_partials_then_reduce_equals_api(product, oracle, torch_gpu, m, n, k, s)
     torch.cuda.synchronize()
     slabs = ws.cpu().numpy().reshape(s, n, m)
     # the API call left the same numbers, by workgroup
-    assert np.array_equal(slabs.view(np.uint16), slabs_from_pages(ws_api.cpu().numpy(), s, m, n).view(np.uint16))
+    assert np.array_equal(slabs.view(np.uint16), slabs_from_pages(ws_api.cpu().numpy(), s, m, n, rows).view(np.uint16))
     for i, (kb, ke) in enumerate(oracle.splitk_ranges(k, s)):
         _, ref = oracle.spmm_model(np.ascontiguousarray(a[:, kb * 64:ke * 64]), np.ascontiguousarray(b_h[:, kb * 64:ke * 64]), n, 1)
         assert_close(slabs[i], ref, f"slab {i}")
@@ -446,6 +480,12 @@ def test_nonuniform_rows(product, oracle, torch_gpu):
 
 
 # --- config 5 flavour: the four linears of a decoder layer, chained --------------------------------
+def test_decoder_layer_chain_eight_row_tile_workgroups(product, oracle, torch_gpu, eight_row_tiles):
+    """64 tokens at hidden 1024 through the eight-wave workgroups of N = 64, the attention-output linear with B read
+    in place at leading dimension 3072."""
+    test_decoder_layer_chain(product, oracle, torch_gpu, 64, 1024)
+
+
 @pytest.mark.parametrize("tokens,hidden", [(16, 512), (256, 512), (64, 1024)])
 def test_decoder_layer_chain(product, oracle, torch_gpu, tokens, hidden):
     """QKV -> (first hidden rows) -> attention output -> FFN1 -> ReLU -> FFN2 on one stream with one

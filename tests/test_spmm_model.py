@@ -102,11 +102,15 @@ def test_slab_page_layout_helper_is_a_bijection_with_known_corners():
     a permutation of the S*N*M halfs, and a few entries placed by hand from the layout's description."""
     from gpu_util import slab_pages, slabs_from_pages
 
-    for m, n, s in [(128, 8, 2), (1024, 16, 7), (1408, 64, 3), (256, 256, 11), (384, 128, 3), (1024, 64, 3), (2048, 32, 5), (512, 32, 2), (1536, 64, 4)]:
+    for m, n, s in [(128, 8, 2), (1024, 16, 7), (1408, 64, 3), (256, 256, 11), (384, 128, 3), (1024, 64, 3), (2048, 32, 5), (512, 32, 2), (1536, 64, 4), (36864, 64, 7)]:
         x = np.arange(s * n * m, dtype=np.int64).reshape(s, n, m)
         p = slab_pages(x, m, n)
         assert np.array_equal(np.sort(p), np.arange(s * n * m))
         assert np.array_equal(slabs_from_pages(p, s, m, n), x)
+        if n == 64 and m % 1024 == 0:   # the layout of workgroups of eight row tiles, whatever their number
+            p = slab_pages(x, m, n, rows=8)
+            assert np.array_equal(np.sort(p), np.arange(s * n * m))
+            assert np.array_equal(slabs_from_pages(p, s, m, n, rows=8), x)
     # M = 1024 (8 row tiles = one per XCD), N = 16, S = 7: unit u, slice sl is workgroup sl*8 + u; its 4 KB page starts
     # at 2048 halfs * workgroup; piece q*64 + g*16 + r = rows 32q+4g.. and 32q+16+4g.. of column r
     m, n, s = 1024, 16, 7
@@ -124,7 +128,7 @@ def test_slab_page_layout_helper_is_a_bijection_with_known_corners():
     # at page sub*G + workgroup
     m, n, s = 2048, 64, 3
     x = np.arange(s * n * m, dtype=np.int64).reshape(s, n, m)
-    p = slab_pages(x, m, n)
+    p = slab_pages(x, m, n, rows=8)
     assert p[0] == x[0, 0, 0]
     assert p[2048 * (1 * 6 + 0)] == x[0, 16, 0]              # sub 1: row tile 0, columns 16..31
     assert p[2048 * (4 * 6 + 0)] == x[0, 0, 128]             # sub 4: row tile 1, columns 0..15

@@ -3,7 +3,7 @@
 kernel_benchmark/benchmark.sh + spmm_test.cu (12 OPT shapes x N x sparsity), for the configurations
 this build is measured on.  Prints one JSON line per case.
 
-    python flash-llm_amd/sweep.py ffn        # FFN shapes, sparsity {70,80,90} %, N {8,16,32,64}
+    python flash-llm_amd/sweep.py ffn        # FFN shapes, sparsity {70,80,90} %, N {8,16,32,64} (and 128, 256 on the up-projection)
     python flash-llm_amd/sweep.py hidden12k  # hidden-12288 projections, Beta(2,8) row densities, N = 32
     python flash-llm_amd/sweep.py square     # 9216 x 9216, N = 16, Split_K {1,2,4,8,heuristic}
     python flash-llm_amd/sweep.py layers     # four chained linears per layer, hidden 9216, 16 tokens, 8 layers
@@ -101,8 +101,9 @@ def main():
         for (m, k) in ((36864, 9216), (9216, 36864)):
             for sp in (0.7, 0.8, 0.9):
                 a = synth.sparse_matrix(m, k, sp, 0, dist="normal", sigma=0.02, threads=threads)
-                for n in (8, 16, 32, 64) + ((128, 256) if sp == 0.8 and m > k else ()):
-                    run_case(torch, f"ffn {m}x{k} s{int(sp * 100)}", a, n, dense=(sp == 0.8))
+                # N = 128 / 256 (the kernel for wide B) on the up-projection: where the dense library takes over
+                for n in (8, 16, 32, 64) + ((128, 256) if m > k else ()):
+                    run_case(torch, f"ffn {m}x{k} s{int(sp * 100)}", a, n, dense=(sp == 0.8 or n >= 128))
     elif what == "hidden12k":
         for (m, k) in ((36864, 12288), (12288, 12288), (49152, 12288), (12288, 49152)):
             a = synth.sparse_matrix(m, k, 0.8, 0, dist="normal", sigma=0.02, row_beta=True, threads=threads)

@@ -65,6 +65,21 @@ def test_workspace_and_heuristic(product):
     assert product.splitk_heuristic(100, 16, 64) == 1
 
 
+def test_constants_of_the_binding_are_those_of_the_header(product):
+    """The Python binding restates a few #defines; they must be the header's values."""
+    text = open(os.path.join(ROOT, "include", "flashllm_spmm.h")).read()
+
+    def define(name):
+        m = re.search(r"#define\s+" + name + r"\s+\(?([^\n/]*?)\)?\s*(?:/\*.*)?$", text, flags=re.M)
+        assert m, name
+        return eval(m.group(1).replace("u", ""))  # "(32u << 20)", "1u", "-3" ...
+
+    assert product.STATIC_WORKSPACE_MAX_BYTES == define("FLASHLLM_STATIC_WORKSPACE_MAX_BYTES") == 32 << 20
+    assert (product.SLABS_PLAIN, product.SLABS_BY_WORKGROUP) == (define("FLASHLLM_SLABS_PLAIN"), define("FLASHLLM_SLABS_BY_WORKGROUP"))
+    assert (product.ENCODE_NO_ZERO, product.ENCODE_OFFSETS, product.ENCODE_RANGE) == (
+        define("FLASHLLM_ENCODE_NO_ZERO"), define("FLASHLLM_ENCODE_OFFSETS"), define("FLASHLLM_ENCODE_RANGE"))
+
+
 def test_bin_file_export(product, oracle, tmp_path):
     m, k = 256, 192
     a = synth.sparse_matrix(m, k, 0.8, 21)

@@ -23,6 +23,9 @@
 //     k per lane).  Any number of tiles may end inside one chunk (empty tiles,
 //     tiles of a single vector).
 //   * One wave, in-order LDS: no barrier anywhere.
+//   * For N = 64 the same wave program runs eight to a workgroup, one row tile each over the same K slice, and
+//     the workgroup stages B in LDS once for all eight (see the kernel's own comment); the waves meet at one
+//     barrier per two k tiles and are otherwise as independent as before.
 //
 // Waiting for memory.  Every path through a ring stage issues exactly one
 // ring load, so the compiler's wait before a slot is used is the exact

@@ -160,21 +160,22 @@ def main():
     def windows(fn, steps, warmup, repeats):
         """ms per call of `repeats` timed windows of `steps` back-to-back calls each, after one settle phase and
         `warmup` untimed calls (the reference times one window of 10 000 launches after 100 warm-ups,
-        kernel_benchmark/spmm_test_utils.h:21-22; several shorter windows show the spread as well)."""
+        kernel_benchmark/spmm_test_utils.h:21-22; several shorter windows show the spread as well).  The whole
+        timed region is bracketed by a synchronize on both sides; inside it the windows follow each other on the
+        stream, separated only by the events that delimit them, so that none but the first starts on an idle GPU
+        (with windows of 20 calls a start from idle costs each call of the window about 0.7 us)."""
         settle(fn)
         for i in range(warmup):
             fn(i)
         torch.cuda.synchronize()
-        out = []
-        for _ in range(repeats):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(repeats + 1)]
+        marks[0].record()
+        for r in range(repeats):
             for i in range(steps):
                 fn(i)
-            e1.record()
-            torch.cuda.synchronize()
-            out.append(e0.elapsed_time(e1) / steps)
-        return sorted(out)
+            marks[r + 1].record()
+        torch.cuda.synchronize()
+        return sorted(marks[r].elapsed_time(marks[r + 1]) / steps for r in range(repeats))
 
     def timed(fn, steps, warmup):
         return windows(fn, steps, warmup, 1)[0]

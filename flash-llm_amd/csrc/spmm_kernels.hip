@@ -71,24 +71,46 @@ constexpr int kLanes     = 64;
 constexpr int kNoTile    = 0x7fffffff;
 constexpr int kXcds      = 8;  // accelerator dies of an MI355X, each with its own L2
 
-// Workgroup w of a launch -> (unit, part), part in [0, parts): the parts of one unit go to workgroups
-// kXcds apart (one XCD under round-robin hand-out), XCD x takes the units x*per_xcd .. (x+1)*per_xcd-1;
-// units beyond a multiple of kXcds are laid out plainly behind them.
-__device__ __forceinline__ void unit_of_workgroup(unsigned w, unsigned units, unsigned parts, int& unit, int& part)
+// Workgroup w of a launch <-> (unit, part), part in [0, parts): the parts of one unit go to workgroups kXcds
+// apart (one XCD under round-robin hand-out), XCD x takes the units x*per_xcd .. (x+1)*per_xcd-1 with
+// per_xcd = units / kXcds:  w = ((unit % per_xcd)*parts + part)*kXcds + unit / per_xcd;  the units beyond a
+// multiple of kXcds are laid out plainly behind them, w = unit*parts + part.
+// The launches are three-dimensional grids (kXcds, parts, layers), whose workgroups the dispatcher hands out in
+// the order x fastest, then y, then z, so that w = x + kXcds*(y + parts*z) and unit and part fall out of the
+// workgroup's coordinates without a division: layer z < per_xcd holds unit x*per_xcd + z, part y.  One more
+// layer holds the units beyond a multiple of kXcds (and a few workgroups that find nothing to do).
+struct Place {
+    int      unit, part;
+    unsigned w;      // position in the launch order described above
+    bool     valid;  // false: a workgroup of the last layer beyond the last unit
+};
+
+__device__ __forceinline__ Place place_of_workgroup(unsigned units, unsigned parts)
 {
     const unsigned per_xcd = units / kXcds;
-    if (w < per_xcd * kXcds * parts) {
-        const unsigned j = w / kXcds;
-        unit             = static_cast<int>((w % kXcds) * per_xcd + j / parts);
-        part             = static_cast<int>(j % parts);
+    Place          p;
+    if (blockIdx.z < per_xcd) {
+        p.unit  = static_cast<int>(blockIdx.x * per_xcd + blockIdx.z);
+        p.part  = static_cast<int>(blockIdx.y);
+        p.w     = blockIdx.x + kXcds * (blockIdx.y + parts * blockIdx.z);
+        p.valid = true;
     }
     else {
-        unit = static_cast<int>(w / parts);
-        part = static_cast<int>(w % parts);
+        const unsigned i = blockIdx.x + kXcds * blockIdx.y;
+        p.unit           = static_cast<int>(per_xcd * kXcds + i / parts);
+        p.part           = static_cast<int>(i % parts);
+        p.w              = per_xcd * kXcds * parts + i;
+        p.valid          = static_cast<unsigned>(p.unit) < units;
     }
+    return p;
 }
 
-// The inverse: which workgroup of the launch has (unit, part).
+inline dim3 grid_of(unsigned units, unsigned parts)
+{
+    return dim3(kXcds, parts, units / kXcds + (units % kXcds ? 1 : 0));
+}
+
+// Which workgroup of the launch has (unit, part).
 __device__ __forceinline__ unsigned workgroup_of_unit(unsigned unit, unsigned part, unsigned units, unsigned parts)
 {
     const unsigned per_xcd = units / kXcds;
@@ -100,17 +122,17 @@ __device__ __forceinline__ unsigned workgroup_of_unit(unsigned unit, unsigned pa
 // Slab storage by workgroup ("pages").  A page is one 128-row x 16-column block of partial sums (4 KB; 128 x 8
 // and 2 KB when N == 8), kept in the order the matrix cores leave it in registers: 16-byte piece
 // q*(4*cols) + g*cols + r16 holds rows 32q + 4g .. +3 and 32q + 16 + 4g .. +3 of column r16.  Page b of
-// workgroup w of a launch of G workgroups is page b*G + w of the workspace.  Under round-robin hand-out the
+// workgroup w (its position in the launch order above) of a launch of G workgroups is page b*G + w of the workspace.  Under round-robin hand-out the
 // XCD that writes and later sums a page is (page index) % 8 whenever G is a multiple of 8, whatever the shape
 // of the product: a workspace shared by the linears of a layer keeps every line in one L2, where stores to
 // lines already present stay readable for the reduction kernel (stores that miss go to memory and do not).
 template<int NBLK>
-__device__ __forceinline__ void store_pages(_Float16* ws, const floatx4 (&acc)[NBLK][8], int first_page, int N, int lane)
+__device__ __forceinline__ void store_pages(_Float16* ws, const floatx4 (&acc)[NBLK][8], int first_page, int N, int lane, unsigned w, unsigned launch)
 {
     const int    cols  = N < 16 ? 8 : 16;
     const int    r16   = lane & 15, g = lane >> 4;
-    const size_t pitch = static_cast<size_t>(gridDim.x) * (cols * 16);  // uint4 between consecutive pages of a workgroup
-    uint4*       page  = reinterpret_cast<uint4*>(ws) + (static_cast<size_t>(first_page) * gridDim.x + blockIdx.x) * (cols * 16);
+    const size_t pitch = static_cast<size_t>(launch) * (cols * 16);  // uint4 between consecutive pages of a workgroup
+    uint4*       page  = reinterpret_cast<uint4*>(ws) + (static_cast<size_t>(first_page) * launch + w) * (cols * 16);
     if (r16 >= cols)
         return;
 #pragma unroll
@@ -269,7 +291,8 @@ __global__ __launch_bounds__(kLanes* W) void spmm_stream_kernel(const uint4* __r
                                                                 int K,
                                                                 int split_k,
                                                                 int col_groups,
-                                                                int pages)
+                                                                int pages,
+                                                                unsigned units)
 {
     constexpr int kBTile  = NB * 2048;                     // bytes of B per k tile in LDS: 16*NB columns x 128
     constexpr int kBBytes = W > 1 ? 2 * G * kBTile : 0;    // two windows
@@ -287,8 +310,10 @@ __global__ __launch_bounds__(kLanes* W) void spmm_stream_kernel(const uint4* __r
     const int kt   = K / kTileCols;
     // W == 1: unit = (row tile, column group), column group fastest: the column groups of a row tile read the
     // same weights and meet in one L2.  W > 1: unit = W consecutive row tiles, all 16*NB columns.
-    int unit, slice;
-    unit_of_workgroup(blockIdx.x, gridDim.x / split_k, split_k, unit, slice);
+    const Place place = place_of_workgroup(units, split_k);
+    if (!place.valid)
+        return;
+    const int  unit = place.unit, slice = place.part;
     const int  rowtile   = W > 1 ? unit * W + wave : unit / col_groups;
     const int  col0      = W > 1 ? 0 : (unit % col_groups) * (16 * NB);
     const bool have_rows = W == 1 || rowtile < M / kTileRows;
@@ -500,7 +525,7 @@ __global__ __launch_bounds__(kLanes* W) void spmm_stream_kernel(const uint4* __r
         return;
     // D layout of the 16x16 MFMA: lane holds column r16, rows 4*g .. 4*g+3 of each 16-row block.
     if (pages) {  // a workgroup's pages: wave by wave, NB each
-        store_pages<NB>(out, acc, wave * NB, N, lane);
+        store_pages<NB>(out, acc, wave * NB, N, lane, place.w, units * split_k);
         return;
     }
     _Float16* o = out + static_cast<size_t>(slice) * M * N + static_cast<size_t>(rowtile) * kTileRows + g * 4;
@@ -557,7 +582,9 @@ __device__ __forceinline__ void spmm_group_body(uint16_t (&tiles)[3][kTileHalfs]
                                                 int ke,
                                                 int col0,
                                                 int vmax,
-                                                int pages)
+                                                int pages,
+                                                unsigned w,
+                                                unsigned launch)
 {
     const int lane = threadIdx.x & (kLanes - 1);
     const int wave = threadIdx.x / kLanes;
@@ -712,7 +739,7 @@ __device__ __forceinline__ void spmm_group_body(uint16_t (&tiles)[3][kTileHalfs]
     int lane_again = threadIdx.x & (kLanes - 1);
     asm volatile("" : "+v"(lane_again));
     if (pages) {  // o is the workspace itself here; this wave's NBW pages follow those of the waves before it
-        store_pages<NBW>(o, acc, static_cast<int>(threadIdx.x / kLanes) * NBW, N, lane_again);
+        store_pages<NBW>(o, acc, static_cast<int>(threadIdx.x / kLanes) * NBW, N, lane_again, w, launch);
         return;
     }
     const int r16 = lane_again & 15, g = lane_again >> 4;
@@ -744,12 +771,15 @@ __global__ __launch_bounds__(kGroupThreads, 3) void spmm_group_kernel(const uint
                                                                   int K,
                                                                   int split_k,
                                                                   int col_groups,
-                                                                  int pages)
+                                                                  int pages,
+                                                                  unsigned units)
 {
     __shared__ __attribute__((aligned(16))) uint16_t tiles[3][kTileHalfs];
-    const int kt = K / kTileCols;
-    int       unit, slice;
-    unit_of_workgroup(blockIdx.x, gridDim.x / split_k, split_k, unit, slice);
+    const int   kt    = K / kTileCols;
+    const Place place = place_of_workgroup(units, split_k);
+    if (!place.valid)
+        return;
+    const int unit = place.unit, slice = place.part;
     const int rowtile = unit / col_groups;
     const int col0    = (unit % col_groups) * (kGroupWaves * 16 * NBW) + (threadIdx.x / kLanes) * (16 * NBW);
     // the reference's slicing (csrc/SpMM_Kernel.cuh:196-204), clamped to K
@@ -771,9 +801,9 @@ __global__ __launch_bounds__(kGroupThreads, 3) void spmm_group_kernel(const uint
     if (whole == 0)
         comp = reinterpret_cast<const uint4*>(B);
     if (whole <= 440LL * (M / kTileRows) * kt)
-        spmm_group_body<NBW, 2>(tiles, comp, toff, B, ldb, o, M, N, K, kb, ke, col0, vmax, pages);
+        spmm_group_body<NBW, 2>(tiles, comp, toff, B, ldb, o, M, N, K, kb, ke, col0, vmax, pages, place.w, units * split_k);
     else
-        spmm_group_body<NBW, 3>(tiles, comp, toff, B, ldb, o, M, N, K, kb, ke, col0, vmax, pages);
+        spmm_group_body<NBW, 3>(tiles, comp, toff, B, ldb, o, M, N, K, kb, ke, col0, vmax, pages, place.w, units * split_k);
 }
 
 __device__ __forceinline__ void add_slab(float (&s)[4], const uint2 v)
@@ -850,25 +880,28 @@ __global__ __launch_bounds__(256) void splitk_reduce_pages_kernel(_Float16* __re
                                                                  int pages_per_unit,
                                                                  int rows_per_unit,
                                                                  int col_groups,
-                                                                 unsigned spmm_grid)
+                                                                 unsigned units)
 {
     const int cols = N < 16 ? 8 : 16;
     const int t    = threadIdx.x;
     if (t >= cols * 16)  // N == 8: half a block
         return;
-    const unsigned units = gridDim.x / pages_per_unit;
-    int            unit, sub;
-    unit_of_workgroup(blockIdx.x, units, pages_per_unit, unit, sub);
-    if ((unit / col_groups) * rows_per_unit + sub / (pages_per_unit / rows_per_unit) >= M / kTileRows)
-        return;  // a row tile beyond the last one (the last unit of a launch may be short of row tiles)
+    const Place place = place_of_workgroup(units, pages_per_unit);
+    if (!place.valid)
+        return;
+    const int      unit = place.unit, sub = place.part;
+    const unsigned spmm_grid = units * split_k;
     const uint4* first = ws + static_cast<size_t>(sub) * spmm_grid * (cols * 16) + t;
-    float        s[8]  = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    // the SpMM launch's workgroup of (unit, slice) is base_w + slice*step_w (workgroup_of_unit, linear in the slice)
+    const unsigned base_w = workgroup_of_unit(unit, 0, units, split_k);
+    const unsigned step_w = static_cast<unsigned>(unit) < units / kXcds * kXcds ? kXcds : 1;
+    float          s[8]   = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int k0 = 0; k0 < split_k; k0 += 8) {
         uint4 v[8];
 #pragma unroll
         for (int j = 0; j < 8; j++)
             if (k0 + j < split_k)
-                v[j] = first[static_cast<size_t>(workgroup_of_unit(unit, k0 + j, units, split_k)) * (cols * 16)];
+                v[j] = first[static_cast<size_t>(base_w + (k0 + j) * step_w) * (cols * 16)];
 #pragma unroll
         for (int j = 0; j < 8; j++)
             if (k0 + j < split_k) {
@@ -895,11 +928,13 @@ __global__ __launch_bounds__(256) void splitk_reduce_pages_kernel(_Float16* __re
     *reinterpret_cast<half4*>(o + 16) = hi;
 }
 
-// out[w] = id of the XCD that workgroup w of this launch ran on
-__global__ __launch_bounds__(kLanes) void xcd_probe_kernel(unsigned* __restrict__ out)
+// out[w] = id of the XCD that workgroup w of this launch ran on, w = x + 8*(y + 3*z) in a grid (8, 3, layers):
+// the order in which the launches above count on their workgroups being handed out
+__global__ __launch_bounds__(kLanes) void xcd_probe_kernel(unsigned* __restrict__ out, unsigned workgroups)
 {
-    if (threadIdx.x == 0)
-        out[blockIdx.x] = __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11));  // XCC_ID, bits 3:0
+    const unsigned w = blockIdx.x + kXcds * (blockIdx.y + 3 * blockIdx.z);
+    if (threadIdx.x == 0 && w < workgroups)
+        out[w] = __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11));  // XCC_ID, bits 3:0
 }
 
 __global__ __launch_bounds__(256) void relu_kernel(uint4* __restrict__ x, long n8)
@@ -926,10 +961,9 @@ __global__ __launch_bounds__(256) void take_rows_kernel(uint4* __restrict__ dst,
 template<int NB, int DEPTH, int W, int G>
 int launch_spmm(hipStream_t stream, const void* comp, const int* offs, const void* b, int ldb, void* out, int m, int n, int k, int split_k, int col_groups, int pages)
 {
-    const unsigned row_units = (static_cast<unsigned>(m / kTileRows) + W - 1) / W;
-    const dim3     grid(row_units * col_groups * split_k, 1, 1);
+    const unsigned units = (static_cast<unsigned>(m / kTileRows) + W - 1) / W * col_groups;
     hipLaunchKernelGGL((spmm_stream_kernel<NB, DEPTH, W, G>),
-                       grid,
+                       grid_of(units, split_k),
                        dim3(kLanes * W),
                        0,
                        stream,
@@ -943,7 +977,8 @@ int launch_spmm(hipStream_t stream, const void* comp, const int* offs, const voi
                        k,
                        split_k,
                        col_groups,
-                       pages);
+                       pages,
+                       units);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -1032,10 +1067,10 @@ extern "C" int flashllm_hip_launch_spmm_group(
     void* stream, const void* comp, const int* offs, const void* b, int ldb, void* out, int m, int n, int k, int split_k, int pages)
 {
     // 128 columns per workgroup (four waves x 32); requires n % 128 == 0
-    const dim3 grid(static_cast<unsigned>(m / kTileRows) * (n / 128) * split_k, 1, 1);
-    hipLaunchKernelGGL(spmm_group_kernel<2>, grid, dim3(kGroupThreads), 0, static_cast<hipStream_t>(stream),
+    const unsigned units = static_cast<unsigned>(m / kTileRows) * (n / 128);
+    hipLaunchKernelGGL(spmm_group_kernel<2>, grid_of(units, split_k), dim3(kGroupThreads), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint4*>(comp), offs, static_cast<const _Float16*>(b), ldb, static_cast<_Float16*>(out),
-                       m, n, k, split_k, n / 128, pages && split_k > 1);
+                       m, n, k, split_k, n / 128, pages && split_k > 1, units);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -1062,22 +1097,24 @@ extern "C" int flashllm_hip_launch_reduce_pages(void* stream, void* c, const voi
     const int      blocks     = group ? 8 : (n <= 16 ? 1 : (n == 32 ? 2 : 4));
     const int      col_groups = group ? n / 128 : (n <= 64 ? 1 : n / 64);
     const unsigned units      = (static_cast<unsigned>(m / kTileRows) + rows - 1) / rows * col_groups;
-    const dim3     grid(units * blocks * rows);
+    const int      pages_per_unit = blocks * rows;
+    const dim3     grid = grid_of(units, pages_per_unit);
     hipStream_t    s  = static_cast<hipStream_t>(stream);
     _Float16*      cp = static_cast<_Float16*>(c);
     const uint4*   wp = static_cast<const uint4*>(ws);
-    const int pages_per_unit = blocks * rows;
-    const unsigned spmm_grid = units * split_k;
     if (relu)
-        hipLaunchKernelGGL(splitk_reduce_pages_kernel<true>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, pages_per_unit, rows, col_groups, spmm_grid);
+        hipLaunchKernelGGL(splitk_reduce_pages_kernel<true>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, pages_per_unit, rows, col_groups, units);
     else
-        hipLaunchKernelGGL(splitk_reduce_pages_kernel<false>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, pages_per_unit, rows, col_groups, spmm_grid);
+        hipLaunchKernelGGL(splitk_reduce_pages_kernel<false>, grid, dim3(256), 0, s, cp, wp, m, n, split_k, pages_per_unit, rows, col_groups, units);
     return static_cast<int>(hipGetLastError());
 }
 
 extern "C" int flashllm_hip_launch_xcd_probe(void* stream, unsigned* out, int workgroups)
 {
-    hipLaunchKernelGGL(xcd_probe_kernel, dim3(workgroups), dim3(kLanes), 0, static_cast<hipStream_t>(stream), out);
+    if (workgroups <= 0)
+        return static_cast<int>(hipErrorInvalidValue);
+    const dim3 grid(kXcds, 3, (static_cast<unsigned>(workgroups) + 3 * kXcds - 1) / (3 * kXcds));
+    hipLaunchKernelGGL(xcd_probe_kernel, grid, dim3(kLanes), 0, static_cast<hipStream_t>(stream), out, static_cast<unsigned>(workgroups));
     return static_cast<int>(hipGetLastError());
 }
 

@@ -64,8 +64,9 @@ int flashllm_hip_launch_reduce(void* stream, void* c, const void* ws, long mn, i
 // and c 8-byte aligned.
 int flashllm_hip_launch_reduce_pages(void* stream, void* c, const void* ws, int m, int n, int split_k, int relu);
 
-// out[w] = id of the XCD workgroup w ran on, for a launch of `workgroups` one-wave workgroups: shows whether
-// the round-robin hand-out the placement above counts on holds on this machine.
+// out[w] = id of the XCD workgroup w ran on, for a launch of `workgroups` one-wave workgroups shaped like the
+// SpMM launches (a three-dimensional grid, eight wide, w counted x first, then y, then z): shows whether the
+// round-robin hand-out in that order, which the placement above counts on, holds on this machine.
 int flashllm_hip_launch_xcd_probe(void* stream, unsigned* out, int workgroups);
 
 // x[i] = max(x[i], 0) over n halfs (n % 8 == 0): the activation between FFN1 and FFN2.

@@ -110,15 +110,6 @@ inline dim3 grid_of(unsigned units, unsigned parts)
     return dim3(kXcds, parts, units / kXcds + (units % kXcds ? 1 : 0));
 }
 
-// Which workgroup of the launch has (unit, part).
-__device__ __forceinline__ unsigned workgroup_of_unit(unsigned unit, unsigned part, unsigned units, unsigned parts)
-{
-    const unsigned per_xcd = units / kXcds;
-    if (unit < per_xcd * kXcds)
-        return ((unit % per_xcd) * parts + part) * kXcds + unit / per_xcd;
-    return unit * parts + part;
-}
-
 // Slab storage by workgroup ("pages").  A page is one 128-row x 16-column block of partial sums (4 KB; 128 x 8
 // and 2 KB when N == 8), kept in the order the matrix cores leave it in registers: 16-byte piece
 // q*(4*cols) + g*cols + r16 holds rows 32q + 4g .. +3 and 32q + 16 + 4g .. +3 of column r16.  Page b of
@@ -892,9 +883,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_pages_kernel(_Float16* __re
     const int      unit = place.unit, sub = place.part;
     const unsigned spmm_grid = units * split_k;
     const uint4* first = ws + static_cast<size_t>(sub) * spmm_grid * (cols * 16) + t;
-    // the SpMM launch's workgroup of (unit, slice) is base_w + slice*step_w (workgroup_of_unit, linear in the slice)
-    const unsigned base_w = workgroup_of_unit(unit, 0, units, split_k);
-    const unsigned step_w = static_cast<unsigned>(unit) < units / kXcds * kXcds ? kXcds : 1;
+    // the SpMM launch's workgroup of (unit, slice) is base_w + slice*step_w (the launch order above is linear in
+    // the part); for a unit of the XCDs' own blocks its two coordinates are this workgroup's x and z
+    const bool     own    = blockIdx.z < units / kXcds;
+    const unsigned base_w = own ? blockIdx.z * split_k * kXcds + blockIdx.x : static_cast<unsigned>(unit) * split_k;
+    const unsigned step_w = own ? kXcds : 1;
     float          s[8]   = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int k0 = 0; k0 < split_k; k0 += 8) {
         uint4 v[8];
@@ -919,7 +912,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_pages_kernel(_Float16* __re
     }
     // piece t = q*(4*cols) + g*cols + r16: rows 32q + 4g .. +3 and 16 further on, column r16 of the block
     // a unit's pages: rows_per_unit row tiles, one after the other, each with the unit's 16-column blocks in order
-    const int q = t / (4 * cols), g = (t / cols) & 3, r16 = t % cols;
+    const int lg = N < 16 ? 3 : 4;  // cols = 1 << lg
+    const int q = t >> (lg + 2), g = (t >> lg) & 3, r16 = t & (cols - 1);
     const int blocks  = pages_per_unit / rows_per_unit;
     const int n       = ((unit % col_groups) * blocks + sub % blocks) * 16 + r16;
     const int rowtile = (unit / col_groups) * rows_per_unit + sub / blocks;

@@ -69,6 +69,8 @@ int flashllm_spmm_splitk(void*       stream,
  * on stderr, before anything is launched.  All calls on one GPU share the array: calls that overlap
  * on one GPU (different streams or threads) race on the slabs; calls on one stream are ordered and safe.
  * Every slab is fully written before it is read, so nothing needs clearing between calls.
+ * The first call on a GPU looks the array's address up (hipGetSymbolAddress) and keeps it; a caller that
+ * records calls under stream capture should make one call outside the capture first.
  */
 #define FLASHLLM_STATIC_WORKSPACE_MAX_BYTES (32u << 20)
 int flashllm_spmm_splitk_static(void*       stream,

@@ -131,12 +131,28 @@ def main():
                 cur, _ = l.forward(cur, tokens, buffers=bufs, workspace=wsp)
 
         ms = timed(torch, all_layers, steps=50)
+        # the same chain recorded once into a HIP graph and replayed (the calls allocate nothing and never wait)
+        all_layers(0)
+        torch.cuda.synchronize()
+        eager = bufs[4].clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            cur = x
+            for l in built:
+                cur, _ = l.forward(cur, tokens, buffers=bufs, workspace=wsp, stream=torch.cuda.current_stream())
+        bufs[4].fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(bufs[4].view(torch.int16), eager.view(torch.int16)), "graph replay differs from the eager chain"
+        ms_graph = timed(torch, lambda i: graph.replay(), steps=50)
         per_layer = []
         for l in built:
             per_layer.append(timed(torch, lambda i: l.forward(x, tokens, buffers=bufs, workspace=wsp), steps=100, settle_ms=50))
         flops = layers * sum(2.0 * m * k * tokens for m, k in shapes)
         print(json.dumps({"case": "chained decoder-layer linears", "hidden": hidden, "tokens": tokens, "layers": layers,
-                          "ms_all_layers": ms, "ms_per_layer": per_layer, "tflops": flops / ms / 1e9,
+                          "ms_all_layers": ms, "ms_all_layers_graph_replay": ms_graph, "ms_per_layer": per_layer, "tflops": flops / ms / 1e9,
                           "weight_GB_compressed": comp_bytes / 1e9, "weight_GB_dense": dense_bytes / 1e9,
                           "alg_GBps": comp_bytes / ms / 1e6, "frac_hbm": comp_bytes / ms / 1e6 / HBM_PEAK}), flush=True)
     elif what == "compress":
